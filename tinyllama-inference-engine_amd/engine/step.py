@@ -1,0 +1,155 @@
+"""The step function: one batch of (request, its next tokens) through the model, from the cache.
+
+reference: `ForwardBatch(tokens, positions, kv_slots)` (src/cuda/model.cu:531-725) takes one
+token per sequence, checks batch size, token range, slot range, that positions continue where the
+slot stopped, and that no slot comes twice (:539-561), runs the rows as one batch, returns the
+logits of every row, and moves `next_positions` only after success (:721-723).  Here an entry
+brings any number of next tokens (a portion of a prompt, or one decoded token), the positions are
+the cache manager's, logits come back only for the wanted places, and the request's length moves
+after the step is enqueued.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import ABSENT, CacheManager
+from ..errors import invalid_argument, out_of_bounds
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)    # places among `tokens` whose logits are asked for
+
+
+@dataclass
+class GroupView:
+    """One page group as the kernels see it in this step."""
+    block_table: torch.Tensor      # int32 [sequences, max_blocks]; absent entries hold page 0 and are never read
+    slot_map: torch.Tensor         # int32 [tokens]: cache row of each token
+    max_blocks: int
+
+
+@dataclass
+class StepContext:
+    """Everything a part may need to know about the step, on the device (and on the host)."""
+    num_tokens: int
+    num_seqs: int
+    num_wanted: int
+    max_new: int                   # most tokens any sequence brings
+    max_context: int               # longest sequence after this step
+    tokens: torch.Tensor           # int32 [T]
+    positions: torch.Tensor        # int32 [T] absolute position of each token in its sequence
+    token_seq: torch.Tensor        # int32 [T] index of the token's sequence in this step
+    no_slots: torch.Tensor         # int32 [T] of -1: a slot map that writes nothing
+    seq_start: torch.Tensor        # int32 [S + 1] first token of each sequence among the T
+    seq_first_pos: torch.Tensor    # int32 [S] position of its first token
+    seq_len: torch.Tensor          # int32 [S] length after this step
+    seq_slot: torch.Tensor         # int32 [S] request slot (row of the state areas)
+    want_rows: torch.Tensor        # int32 [num_wanted] token indices
+    groups: list[GroupView]
+    host: dict                     # the same arrays as numpy, by name
+
+
+class ModelRunner:
+    def __init__(self, model, cache: CacheManager):
+        self.model = model
+        self.cache = cache
+        self.device = model.device
+        self.vocab_size = model.spec.vocab_size
+
+    # ---- checks and context ------------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise invalid_argument("a step needs at least one entry")
+        seen = set()
+        for entry in entries:
+            if entry.request in seen:
+                raise invalid_argument(f"request {entry.request!r} comes twice in one step")
+            seen.add(entry.request)
+            if len(entry.tokens) == 0:
+                raise invalid_argument(f"request {entry.request!r} brings no tokens")
+            for token in entry.tokens:
+                if not 0 <= int(token) < self.vocab_size:
+                    raise out_of_bounds(f"token {token} of request {entry.request!r} is outside the vocabulary of {self.vocab_size}")
+            for place in entry.want:
+                if not 0 <= int(place) < len(entry.tokens):
+                    raise out_of_bounds(f"wanted place {place} of request {entry.request!r} is not among its {len(entry.tokens)} tokens")
+            if not self.cache.is_live(entry.request):
+                raise invalid_argument(f"request {entry.request!r} is not live (admit it first)")
+            limit = self.cache.max_positions
+            if limit is not None and self.cache.length(entry.request) + len(entry.tokens) > limit:
+                raise out_of_bounds(f"request {entry.request!r} would pass the model's {limit} positions")
+
+    def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
+        cache = self.cache
+        counts = [len(entry.tokens) for entry in entries]
+        total, seqs = sum(counts), len(entries)
+        first = [cache.length(entry.request) for entry in entries]
+        tokens = np.concatenate([np.asarray(entry.tokens, dtype=np.int32) for entry in entries])
+        positions = np.concatenate([np.arange(start, start + n, dtype=np.int32) for start, n in zip(first, counts)])
+        token_seq = np.repeat(np.arange(seqs, dtype=np.int32), counts)
+        seq_start = np.zeros(seqs + 1, dtype=np.int32)
+        seq_start[1:] = np.cumsum(counts)
+        want_rows = np.asarray([seq_start[index] + int(place) for index, entry in enumerate(entries) for place in entry.want],
+                               dtype=np.int32)
+        host = {
+            "tokens": tokens, "positions": positions, "token_seq": token_seq,
+            "no_slots": np.full(total, -1, dtype=np.int32), "seq_start": seq_start,
+            "seq_first_pos": np.asarray(first, dtype=np.int32),
+            "seq_len": np.asarray([start + n for start, n in zip(first, counts)], dtype=np.int32),
+            "seq_slot": np.asarray([cache.slot(entry.request) for entry in entries], dtype=np.int32),
+            "want_rows": want_rows,
+        }
+        group_shapes = []
+        for group in range(len(cache.groups)):
+            lists = [cache.page_list(entry.request, group) for entry in entries]
+            width = max(1, max(len(pages) for pages in lists))
+            table = np.zeros((seqs, width), dtype=np.int32)
+            for row, pages in enumerate(lists):
+                table[row, :len(pages)] = [page if page != ABSENT else 0 for page in pages]
+            slot_map = np.concatenate([np.asarray(cache.rows(entry.request, group, start, n), dtype=np.int32)
+                                       for entry, start, n in zip(entries, first, counts)])
+            host[f"block_table{group}"] = table
+            host[f"slot_map{group}"] = slot_map
+            group_shapes.append(width)
+        # one transfer for all of it
+        names = list(host)
+        flat = np.concatenate([host[name].ravel() for name in names])
+        device_flat = torch.from_numpy(flat).to(self.device, non_blocking=False)
+        views, cursor = {}, 0
+        for name in names:
+            size = host[name].size
+            views[name] = device_flat[cursor:cursor + size].view(host[name].shape)
+            cursor += size
+        groups = [GroupView(views[f"block_table{group}"], views[f"slot_map{group}"], width)
+                  for group, width in enumerate(group_shapes)]
+        return StepContext(
+            num_tokens=total, num_seqs=seqs, num_wanted=int(want_rows.size), max_new=max(counts),
+            max_context=int(host["seq_len"].max()), tokens=views["tokens"], positions=views["positions"],
+            token_seq=views["token_seq"], no_slots=views["no_slots"], seq_start=views["seq_start"],
+            seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
+            want_rows=views["want_rows"], groups=groups, host=host)
+
+    # ---- the step ----------------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Runs exactly the tokens the entries bring, as one batch, from the cache that earlier
+        steps left.  Returns float32 logits [wanted places, vocab] on the device, in the order of
+        the entries and of each entry's `want`."""
+        self._validate(entries)
+        wanted = [(entry.request, len(entry.tokens)) for entry in entries]
+        if not self.cache.can_reserve(wanted):
+            from ..errors import out_of_memory
+            raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
+        for request, count in wanted:
+            self.cache.reserve(request, count)
+        ctx = self.build_context(entries)
+        logits = self.model.forward(ctx, self.cache.bindings)
+        for request, count in wanted:
+            self.cache.commit(request, count)
+        return logits

@@ -1,0 +1,70 @@
+"""From a `ModelSpec` to a model that runs: the parts are looked up by kind and built with their
+own parameters; nothing here names an architecture."""
+from __future__ import annotations
+
+import torch
+
+from .. import parts as _parts  # noqa: F401  (fills the part registries)
+from ..cache.manager import RunNeed
+from ..config.spec import ModelSpec, TensorSpec
+from ..registry import lookup
+
+
+def expected_tensors(spec: ModelSpec) -> list[TensorSpec]:
+    """Every tensor the model's parts expect, by full name; the list that weights are checked
+    against and that random weights are drawn for (the reference's fixed list of 9 per layer + 3
+    is `ExpectedTensors`, src/model_config.cpp:78-97)."""
+    specs = list(lookup("embedding", spec.embedding.kind).tensor_specs(spec.embedding, ""))
+    for layer in spec.layers:
+        specs += lookup("block", layer.block).tensor_specs(layer)
+    specs += lookup("norm", spec.final_norm.kind).tensor_specs(spec.final_norm, "model.norm.")
+    specs += lookup("head", spec.head.kind).tensor_specs(spec.head, "")
+    names = [tensor.name for tensor in specs]
+    if len(set(names)) != len(names):
+        raise AssertionError("two parts claim the same tensor name")
+    return specs
+
+
+class DecoderModel:
+    """Embedding, the layers in the order of `spec.runs`, final norm at the wanted rows, head."""
+
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, device):
+        spec.validate()
+        self.spec = spec
+        self.dtype = dtype
+        self.device = device
+        self.embedding = lookup("embedding", spec.embedding.kind)(spec.embedding, dtype, device)
+        self.blocks = [lookup("block", layer.block)(layer, dtype, device) for layer in spec.layers]
+        self.final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, dtype, device)
+        self.head = lookup("head", spec.head.kind)(spec.head, dtype, device)
+
+    def load(self, weights: dict[str, torch.Tensor]) -> None:
+        self.embedding.load(weights, "")
+        for block in self.blocks:
+            block.load(weights)
+        self.final_norm.load(weights, "model.norm.")
+        self.head.load(weights, "")
+
+    def run_needs(self) -> list[RunNeed]:
+        needs = []
+        for run in self.spec.runs:
+            mixer = self.blocks[run.layer].mixer
+            needs.append(RunNeed(cache_of=run.cache_of, kv=mixer.cache_need(), state=mixer.state_need()))
+        return needs
+
+    def forward(self, ctx, bindings) -> torch.Tensor:
+        """Runs the step's tokens; returns float32 logits [wanted rows, vocab]."""
+        residual = self.embedding.forward(ctx.tokens)
+        pending = None
+        for index, run in enumerate(self.spec.runs):
+            pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index])
+        if ctx.num_wanted == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        normed = self.final_norm.add_forward(residual, pending, rows=ctx.want_rows)
+        return self.head.forward(normed)
+
+
+def build_model(spec: ModelSpec, weights: dict[str, torch.Tensor], dtype: torch.dtype, device) -> DecoderModel:
+    model = DecoderModel(spec, dtype, device)
+    model.load(weights)
+    return model

@@ -1,0 +1,258 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that operand shapes, types and index ranges are what the kernel
+and its grid assume, raises `EngineError` when they are not, and only then launches on torch's
+current stream.  Nothing here computes anything in torch: without the compiled library (and a
+GPU) these functions fail.
+"""
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from .csrc import build as _build
+from .errors import EngineError, ErrorCode, invalid_argument, invalid_shape
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    if dtype not in _CODES:
+        raise EngineError(ErrorCode.INVALID_DTYPE, f"kernels take float32 or bfloat16, not {dtype}")
+    return _CODES[dtype]
+
+
+def library() -> ctypes.CDLL:
+    return _build.load()
+
+
+def _ptr(tensor: torch.Tensor | None):
+    return ctypes.c_void_p(tensor.data_ptr()) if tensor is not None else ctypes.c_void_p(0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(status: int, what: str) -> None:
+    if status == 0:
+        return
+    if status == -1:
+        raise invalid_argument(f"{what}: the kernel does not take these sizes or types")
+    raise EngineError(ErrorCode.HIP, f"{what}: the launch failed (status {status})")
+
+
+def _device_tensor(tensor: torch.Tensor, name: str, dtype: torch.dtype | tuple | None = None) -> None:
+    if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda:
+        raise invalid_argument(f"{name} must be a tensor on the GPU")
+    if not tensor.is_contiguous():
+        raise invalid_argument(f"{name} must be contiguous")
+    if dtype is not None:
+        allowed = dtype if isinstance(dtype, tuple) else (dtype,)
+        if tensor.dtype not in allowed:
+            raise EngineError(ErrorCode.INVALID_DTYPE, f"{name} has dtype {tensor.dtype}, expected one of {allowed}")
+
+
+@dataclass
+class Product:
+    """The result of a matrix product: [rows, cols], or `nsplit` float partial sums
+    [nsplit, rows, cols] of a split-K kernel that the consumer adds up."""
+    data: torch.Tensor
+    nsplit: int = 1
+
+    @property
+    def rows(self) -> int:
+        return self.data.shape[-2]
+
+    @property
+    def cols(self) -> int:
+        return self.data.shape[-1]
+
+    @property
+    def split_stride(self) -> int:
+        return self.rows * self.cols
+
+    def dense(self, dtype: torch.dtype | None = None) -> torch.Tensor:
+        """The summed result as one tensor (for parts that do not fuse the sum)."""
+        out = self.data if self.nsplit == 1 and self.data.dim() == 2 else self.data.view(self.nsplit, self.rows, self.cols).sum(0)
+        return out if dtype is None or out.dtype == dtype else out.to(dtype)
+
+
+def as_product(value) -> Product:
+    if isinstance(value, Product):
+        return value
+    if isinstance(value, torch.Tensor) and value.dim() == 2:
+        return Product(value.contiguous(), 1)
+    raise invalid_argument("a part must return a [tokens, width] tensor or a Product")
+
+
+def _check_product(product: Product, name: str) -> None:
+    _device_tensor(product.data, name, (torch.float32, torch.bfloat16))
+    if product.nsplit < 1 or product.data.numel() != product.nsplit * product.rows * product.cols:
+        raise invalid_shape(f"{name}: {product.nsplit} splits do not fit a tensor of shape {list(product.data.shape)}")
+    if product.nsplit > 1 and product.data.dtype != torch.float32:
+        raise EngineError(ErrorCode.INVALID_DTYPE, f"{name}: partial sums must be float32")
+
+
+# ---------------------------------------------------------------------------------------------
+def embed_gather(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """float32 residual[t, :] = table[tokens[t], :].  The caller has checked 0 <= token < vocab."""
+    _device_tensor(tokens, "tokens", torch.int32)
+    _device_tensor(table, "embedding table", (torch.float32, torch.bfloat16))
+    if tokens.dim() != 1 or table.dim() != 2:
+        raise invalid_shape("embed_gather takes tokens [T] and a table [vocab, hidden]")
+    out = torch.empty((tokens.shape[0], table.shape[1]), dtype=torch.float32, device=table.device)
+    _check(library().tlie_embed_gather(_ptr(tokens), _ptr(table), dtype_code(table.dtype), _ptr(out),
+                                       tokens.shape[0], table.shape[1], _stream()), "embed_gather")
+    return out
+
+
+def add_rmsnorm(residual: torch.Tensor, delta: Product | None, weight: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: torch.Tensor | None = None, want_out: bool = True) -> torch.Tensor | None:
+    """residual += delta (all rows, in place) and out = RMSNorm(residual) * weight.
+
+    With `rows` (int32 indices) only those rows are normed, from residual + delta, and the
+    residual is left as it was.  `delta` may be None (norm only)."""
+    _device_tensor(residual, "residual", torch.float32)
+    _device_tensor(weight, "norm weight", (torch.float32, torch.bfloat16))
+    if residual.dim() != 2 or weight.shape != (residual.shape[1],):
+        raise invalid_shape(f"add_rmsnorm: residual {list(residual.shape)} and weight {list(weight.shape)} do not fit")
+    if not eps > 0.0:
+        raise EngineError(ErrorCode.NUMERICAL, "RMSNorm requires a positive epsilon")
+    tokens, hidden = residual.shape
+    delta_code, nsplit, stride = F32, 1, 0
+    if delta is not None:
+        _check_product(delta, "delta")
+        if (delta.rows, delta.cols) != (tokens, hidden):
+            raise invalid_shape(f"add_rmsnorm: delta [{delta.rows}, {delta.cols}] does not fit residual {list(residual.shape)}")
+        delta_code, nsplit, stride = dtype_code(delta.data.dtype), delta.nsplit, delta.split_stride
+    count = tokens
+    if rows is not None:
+        _device_tensor(rows, "rows", torch.int32)
+        count = rows.shape[0]
+        if count == 0:
+            return torch.empty((0, hidden), dtype=out_dtype, device=residual.device)
+    out = torch.empty((count, hidden), dtype=out_dtype, device=residual.device) if want_out else None
+    _check(library().tlie_add_rmsnorm(_ptr(residual), _ptr(delta.data if delta is not None else None), delta_code, nsplit,
+                                      ctypes.c_longlong(stride), _ptr(weight), dtype_code(weight.dtype),
+                                      ctypes.c_float(eps), _ptr(out), dtype_code(out_dtype), _ptr(rows), count, hidden,
+                                      _stream()), "add_rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: Product, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i]."""
+    _check_product(gate_up, "gate_up")
+    if gate_up.cols % 2 != 0:
+        raise invalid_shape("silu_mul: the input holds gate and up side by side, its width must be even")
+    rows, inter = gate_up.rows, gate_up.cols // 2
+    out = torch.empty((rows, inter), dtype=out_dtype, device=gate_up.data.device)
+    _check(library().tlie_silu_mul(_ptr(gate_up.data), dtype_code(gate_up.data.dtype), gate_up.nsplit,
+                                   ctypes.c_longlong(gate_up.split_stride), _ptr(out), dtype_code(out_dtype), rows, inter,
+                                   _stream()), "silu_mul")
+    return out
+
+
+def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
+               rot_dim: int, cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+               act_dtype: torch.dtype) -> torch.Tensor:
+    """Rotates q and k, returns q [T, nq * d], writes k and v into the cache rows of `slot_map`.
+
+    cache: [pages, 2, nkv, page_size, d].  slot_map[t] = page * page_size + row, or -1 to skip.
+    The slot map comes from the cache manager, which hands out only rows of pages it owns."""
+    _check_product(qkv, "qkv")
+    _device_tensor(positions, "positions", torch.int32)
+    _device_tensor(slot_map, "slot_map", torch.int32)
+    _device_tensor(cache, "cache", act_dtype)
+    tokens = qkv.rows
+    if qkv.cols != (num_heads + 2 * num_kv_heads) * head_dim:
+        raise invalid_shape(f"rope_cache: qkv width {qkv.cols} is not (nq + 2 nkv) * d")
+    if positions.shape != (tokens,) or slot_map.shape != (tokens,):
+        raise invalid_shape("rope_cache: positions and slot_map need one entry per token")
+    if cache.dim() != 5 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[4] != head_dim:
+        raise invalid_shape(f"rope_cache: cache {list(cache.shape)} is not [pages, 2, nkv, page_size, d]")
+    if inv_freq is not None:
+        _device_tensor(inv_freq, "inv_freq", torch.float32)
+        if rot_dim % 2 != 0 or not 0 < rot_dim <= head_dim or inv_freq.shape != (rot_dim // 2,):
+            raise invalid_shape("rope_cache: inv_freq needs rot_dim / 2 entries, rot_dim even and at most d")
+    else:
+        rot_dim = 0
+    q_out = torch.empty((tokens, num_heads * head_dim), dtype=act_dtype, device=cache.device)
+    _check(library().tlie_rope_cache(_ptr(qkv.data), dtype_code(qkv.data.dtype), qkv.nsplit,
+                                     ctypes.c_longlong(qkv.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
+                                     rot_dim, _ptr(q_out), _ptr(cache), dtype_code(act_dtype), tokens, num_heads,
+                                     num_kv_heads, head_dim, cache.shape[3], _stream()), "rope_cache")
+    return q_out
+
+
+def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, token_seq: torch.Tensor,
+                      positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                      window: int | None, scale: float) -> torch.Tensor:
+    """Causal attention of every token over its sequence's cached keys; any number of tokens per
+    sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it."""
+    _device_tensor(q, "q", (torch.float32, torch.bfloat16))
+    _device_tensor(cache, "cache", q.dtype)
+    _device_tensor(block_table, "block_table", torch.int32)
+    _device_tensor(token_seq, "token_seq", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    tokens = q.shape[0]
+    if q.shape != (tokens, num_heads * head_dim):
+        raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
+    if cache.dim() != 5 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[4] != head_dim:
+        raise invalid_shape(f"attention: cache {list(cache.shape)} is not [pages, 2, nkv, page_size, d]")
+    if block_table.dim() != 2 or token_seq.shape != (tokens,) or positions.shape != (tokens,):
+        raise invalid_shape("attention: block_table must be [sequences, max_blocks], token_seq and positions [tokens]")
+    if num_heads % num_kv_heads != 0:
+        raise invalid_shape("attention: the number of heads must be a multiple of the number of kv heads")
+    out = torch.empty_like(q)
+    _check(library().tlie_attention_generic(_ptr(q), _ptr(cache), dtype_code(q.dtype), _ptr(block_table),
+                                            block_table.shape[1], _ptr(token_seq), _ptr(positions), _ptr(out), tokens,
+                                            num_heads, num_kv_heads, head_dim, cache.shape[3],
+                                            int(window) if window else 0, ctypes.c_float(scale), _stream()),
+           "attention_generic")
+    return out
+
+
+def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out_dtype: torch.dtype) -> Product:
+    """y = x . W^T (+ bias), every product and sum in true 32-bit.  W is [out, in]."""
+    _device_tensor(x, "x", (torch.float32, torch.bfloat16))
+    _device_tensor(weight, "weight", (torch.float32, torch.bfloat16))
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise invalid_shape(f"gemm: x {list(x.shape)} and weight {list(weight.shape)} do not fit")
+    if bias is not None:
+        _device_tensor(bias, "bias", weight.dtype)
+        if bias.shape != (weight.shape[0],):
+            raise invalid_shape("gemm: bias needs one entry per output")
+    out = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=x.device)
+    if x.shape[0] == 0:
+        return Product(out, 1)
+    _check(library().tlie_gemm_generic(_ptr(x), dtype_code(x.dtype), _ptr(weight), dtype_code(weight.dtype), _ptr(bias),
+                                       _ptr(out), dtype_code(out_dtype), x.shape[0], weight.shape[0], x.shape[1],
+                                       _stream()), "gemm_generic")
+    return Product(out, 1)
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
+           seed: torch.Tensor | None = None, counter: torch.Tensor | None = None) -> torch.Tensor:
+    """One token per row of float32 logits: the first maximum when the row's temperature is not
+    positive (or none is given), else a draw from the top-p part of softmax(logits / T) with the
+    uniform number of (seed, counter).  A row with a NaN or an infinity gives -1."""
+    _device_tensor(logits, "logits", torch.float32)
+    if logits.dim() != 2:
+        raise invalid_shape("sample takes logits [rows, vocab]")
+    rows = logits.shape[0]
+    for name, tensor, dtype in (("temperature", temperature, torch.float32), ("top_p", top_p, torch.float32),
+                                ("seed", seed, torch.int64), ("counter", counter, torch.int64)):
+        if tensor is not None:
+            _device_tensor(tensor, name, dtype)
+            if tensor.shape != (rows,):
+                raise invalid_shape(f"sample: {name} needs one entry per row")
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    if rows == 0:
+        return out
+    _check(library().tlie_sample(_ptr(logits), rows, logits.shape[1], _ptr(temperature), _ptr(top_p), _ptr(seed),
+                                 _ptr(counter), _ptr(out), _stream()), "sample")
+    return out

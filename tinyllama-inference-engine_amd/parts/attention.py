@@ -1,0 +1,88 @@
+"""Grouped-query causal attention over the paged cache.
+
+reference (one token at a time, src/model.cpp:140-179; src/cuda/model.cu:412-447): q, k, v
+projections of the normed input; rotation of q and k; the rotated key and the value go to the
+cache at the token's position; each query head h attends over the cached keys 0..pos of kv head
+h // (nq / nkv) with scores scaled by 1/sqrt(d) after the dot product; the output projection
+follows.  Here the three projections are one product over the concatenated weight, the rotation
+and the cache write are one kernel, and all tokens of a step run together.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from .. import ops
+from ..config.spec import PartSpec, TensorSpec
+from ..errors import invalid_config
+from ..registry import lookup, register
+from .base import Binding, KVCacheNeed, Mixer, PositionEncoding
+from .linear import Linear
+
+
+@register("mixer", "attention")
+class Attention(Mixer):
+    """spec: hidden_size, num_heads, num_kv_heads, head_dim, bias, window (None or a count of
+    positions), position (a PartSpec of a position encoding).
+    Tensors: `<prefix>{q,k,v,o}_proj.weight` (and `.bias` when bias)."""
+
+    def __init__(self, spec: PartSpec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.hidden = int(spec["hidden_size"])
+        self.nq = int(spec["num_heads"])
+        self.nkv = int(spec["num_kv_heads"])
+        self.d = int(spec["head_dim"])
+        self.bias = bool(spec.get("bias", False))
+        self.window = spec.get("window")
+        if self.nq % self.nkv != 0:
+            raise invalid_config("attention: num_heads must be a multiple of num_kv_heads")
+        if self.window is not None and int(self.window) <= 0:
+            raise invalid_config("attention: a window must be a positive count of positions")
+        position = spec.get("position") or PartSpec("none")
+        self.position = lookup("position_encoding", position.kind)(position, dtype, device)
+        self.scale = 1.0 / math.sqrt(float(self.d))
+        self.qkv = self.o = None
+
+    @classmethod
+    def tensor_specs(cls, spec, prefix):
+        hidden, d = int(spec["hidden_size"]), int(spec["head_dim"])
+        qd, kvd = int(spec["num_heads"]) * d, int(spec["num_kv_heads"]) * d
+        shapes = (("q_proj", (qd, hidden)), ("k_proj", (kvd, hidden)), ("v_proj", (kvd, hidden)), ("o_proj", (hidden, qd)))
+        specs = [TensorSpec(f"{prefix}{name}.weight", shape) for name, shape in shapes]
+        if spec.get("bias", False):
+            specs += [TensorSpec(f"{prefix}{name}.bias", (shape[0],)) for name, shape in shapes]
+        return specs
+
+    def load(self, weights, prefix):
+        def cat(suffix):
+            return torch.cat([weights[f"{prefix}{name}_proj.{suffix}"] for name in "qkv"], dim=0)
+        self.qkv = Linear(cat("weight"), cat("bias") if self.bias else None, self.dtype)
+        self.o = Linear(weights[prefix + "o_proj.weight"], weights.get(prefix + "o_proj.bias") if self.bias else None,
+                        self.dtype)
+
+    def cache_need(self):
+        return KVCacheNeed(self.nkv, self.d, int(self.window) if self.window is not None else None)
+
+    def forward(self, x, ctx, binding: Binding):
+        pages = ctx.groups[binding.group]
+        qkv = self.qkv(x)
+        slot_map = pages.slot_map if binding.writes else ctx.no_slots
+        table = self.position.rotary_table()
+        if table is None and type(self.position).apply_qk is not PositionEncoding.apply_qk:
+            qkv = self._apply_other_positions(qkv, ctx)
+        inv_freq, rot_dim = table if table is not None else (None, 0)
+        q = ops.rope_cache(qkv, ctx.positions, slot_map, inv_freq, rot_dim, binding.cache, self.nq, self.nkv, self.d,
+                           self.dtype)
+        attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
+                                         self.nkv, self.d, self.window, self.scale)
+        return self.o(attended)
+
+    def _apply_other_positions(self, qkv, ctx):
+        """A position encoding that is no rotation table: applied to q and k as tensors."""
+        dense = qkv.dense(self.dtype)
+        qd, kvd = self.nq * self.d, self.nkv * self.d
+        q, k = self.position.apply_qk(dense[:, :qd].reshape(-1, self.nq, self.d),
+                                      dense[:, qd:qd + kvd].reshape(-1, self.nkv, self.d), ctx.positions)
+        joined = torch.cat([q.reshape(-1, qd), k.reshape(-1, kvd), dense[:, qd + kvd:]], dim=1).contiguous()
+        return ops.Product(joined, 1)

@@ -1,0 +1,110 @@
+"""The interfaces of the parts a model is put together from.
+
+A part is built from its `PartSpec` (sizes and constants), says which tensors it expects under a
+prefix, takes them, and runs on the tokens of one step.  It does not know which model it is in,
+which layer it is, or how the step was cut; what it may need to know about the step (positions,
+which sequence a token belongs to, where its cache rows are) arrives in the `StepContext`, and
+what the cache manager holds for it arrives in the `Binding`.
+
+    Norm           forward(residual f32 [T, H]) -> [T, H] in the activation type
+                   add_forward(residual, delta, rows=None): residual += delta, then forward
+    Mixer          forward(x [T, H], ctx, binding) -> Product or tensor [T, H]
+                   cache_need() -> KVCacheNeed | None;  state_need() -> StateNeed | None
+    FeedForward    forward(x [T, H], ctx) -> Product or tensor [T, H]
+    PositionEncoding
+                   rotary_table() -> (inv_freq, rot_dim) | None   (lets attention fuse it)
+                   apply_qk(q, k, positions) -> (q, k)             (any other scheme)
+    Block          forward(residual, pending, ctx, binding) -> pending
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+
+from ..config.spec import PartSpec, TensorSpec
+from ..ops import Product, as_product
+
+
+@dataclass(frozen=True)
+class KVCacheNeed:
+    """Pages of keys and values: [2, num_kv_heads, page_size, head_dim] per page.  `window`
+    None: every key stays; else only the last `window` positions are ever read again."""
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """State of fixed size per request: one row of `shape` in an area indexed by request slot."""
+    shape: tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class Binding:
+    """What the cache manager holds for one run of a layer."""
+    group: int | None = None            # index of the page group (block table, slot map) in the step context
+    cache: torch.Tensor | None = None   # [pages, 2, nkv, page_size, d] of the run whose cache is read
+    writes: bool = True                 # this run owns the cache and writes the step's keys and values
+    state: torch.Tensor | None = None   # [request slots, *shape] for a mixer with state of its own
+
+
+class Part:
+    def __init__(self, spec: PartSpec, dtype: torch.dtype, device):
+        self.spec = spec
+        self.dtype = dtype              # the activation type: float32 or bfloat16
+        self.device = device
+
+    @classmethod
+    def tensor_specs(cls, spec: PartSpec, prefix: str) -> list[TensorSpec]:
+        return []
+
+    def load(self, weights: dict[str, torch.Tensor], prefix: str) -> None:
+        pass
+
+
+class Norm(Part):
+    def forward(self, residual: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+    def add_forward(self, residual: torch.Tensor, delta, rows: torch.Tensor | None = None) -> torch.Tensor:
+        """Unfused default: add in place, then norm; with `rows`, norm those rows of the sum only."""
+        if rows is not None:
+            picked = residual[rows.long()]
+            if delta is not None:
+                picked = picked + as_product(delta).dense(torch.float32)[rows.long()]
+            return self.forward(picked.contiguous())
+        if delta is not None:
+            residual += as_product(delta).dense(torch.float32)
+        return self.forward(residual)
+
+
+class PositionEncoding(Part):
+    def rotary_table(self):
+        return None
+
+    def apply_qk(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor):
+        return q, k
+
+
+class Mixer(Part):
+    def cache_need(self) -> KVCacheNeed | None:
+        return None
+
+    def state_need(self) -> StateNeed | None:
+        return None
+
+    def forward(self, x: torch.Tensor, ctx: Any, binding: Binding):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x: torch.Tensor, ctx: Any):
+        raise NotImplementedError
+
+
+__all__ = ["KVCacheNeed", "StateNeed", "Binding", "Part", "Norm", "PositionEncoding", "Mixer", "FeedForward",
+           "Product", "as_product"]

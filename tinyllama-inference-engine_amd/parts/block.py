@@ -1,0 +1,46 @@
+"""How a layer's parts are arranged.
+
+"pre_norm" is the reference's block (src/model.cpp:132-203): x += mixer(norm(x)), then
+x += feed_forward(norm(x)); the residual itself is never normed in place.  The residual is a
+float32 array that lives for the whole step.  A block does not add its last result itself: it
+hands it on as `pending`, and whoever norms the residual next (the next block's first norm, or
+the model's final norm) adds it in the same kernel.
+"""
+from __future__ import annotations
+
+from ..config.spec import LayerSpec
+from ..registry import lookup, register
+
+
+@register("block", "pre_norm")
+class PreNormBlock:
+    def __init__(self, layer: LayerSpec, dtype, device):
+        self.layer = layer
+        self.mixer_norm = lookup("norm", layer.mixer_norm.kind)(layer.mixer_norm, dtype, device)
+        self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
+        self.feed_forward_norm = lookup("norm", layer.feed_forward_norm.kind)(layer.feed_forward_norm, dtype, device)
+        self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
+
+    # names under the layer's prefix, as the reference's checkpoints have them
+    # (src/model_config.cpp:81-95)
+    _PLACES = (("mixer_norm", "input_layernorm."), ("mixer", "self_attn."),
+               ("feed_forward_norm", "post_attention_layernorm."), ("feed_forward", "mlp."))
+
+    @classmethod
+    def tensor_specs(cls, layer: LayerSpec):
+        specs = []
+        for attribute, place in cls._PLACES:
+            part_spec = getattr(layer, attribute)
+            table = {"mixer_norm": "norm", "feed_forward_norm": "norm"}.get(attribute, attribute)
+            specs += lookup(table, part_spec.kind).tensor_specs(part_spec, layer.prefix + place)
+        return specs
+
+    def load(self, weights):
+        for attribute, place in self._PLACES:
+            getattr(self, attribute).load(weights, self.layer.prefix + place)
+
+    def forward(self, residual, pending, ctx, binding):
+        normed = self.mixer_norm.add_forward(residual, pending)
+        mixed = self.mixer.forward(normed, ctx, binding)
+        normed = self.feed_forward_norm.add_forward(residual, mixed)
+        return self.feed_forward.forward(normed, ctx)

@@ -1,0 +1,57 @@
+"""The two ends of the model: the token embedding and the output head.
+
+reference: the embedding is a row copy, unscaled (src/model.cpp:94-97); the head is a plain
+product of the final norm's output with `lm_head.weight`, no bias, no scaling
+(src/model.cpp:224-225).  With tied embeddings the head's matrix is the embedding table.
+Logits are float32 whatever the activation type."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from ..config.spec import PartSpec, TensorSpec
+from ..registry import register
+from .base import Part
+from .linear import Linear
+
+
+@register("embedding", "token_embedding")
+class TokenEmbedding(Part):
+    NAME = "model.embed_tokens.weight"
+
+    def __init__(self, spec: PartSpec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.table = None
+
+    @classmethod
+    def tensor_specs(cls, spec, prefix=""):
+        return [TensorSpec(cls.NAME, (int(spec["vocab_size"]), int(spec["hidden_size"])))]
+
+    def load(self, weights, prefix=""):
+        self.table = weights[self.NAME].contiguous()
+
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        return ops.embed_gather(tokens, self.table)
+
+
+@register("head", "lm_head")
+class LMHead(Part):
+    NAME = "lm_head.weight"
+
+    def __init__(self, spec: PartSpec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.tied = bool(spec.get("tied", False))
+        self.linear = None
+
+    @classmethod
+    def tensor_specs(cls, spec, prefix=""):
+        shape = (int(spec["vocab_size"]), int(spec["hidden_size"]))
+        # a tied model may still carry the head's matrix; it is then not read
+        return [TensorSpec(cls.NAME, shape, optional=bool(spec.get("tied", False)))]
+
+    def load(self, weights, prefix=""):
+        matrix = weights[TokenEmbedding.NAME] if self.tied else weights[self.NAME]
+        self.linear = Linear(matrix, None, self.dtype)
+
+    def forward(self, normed: torch.Tensor) -> torch.Tensor:
+        return self.linear(normed, out_dtype=torch.float32).dense(torch.float32)

@@ -1,0 +1,36 @@
+"""RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w (src/operators.cpp:22-45 of the reference; its
+device form, src/cuda/kernels.cu:67-84).  The residual it reads is float32; the sum of squares,
+the scale and the product are float32; the output is in the activation type."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from ..config.spec import PartSpec, TensorSpec
+from ..registry import register
+from .base import Norm, as_product
+
+
+@register("norm", "rms_norm")
+class RMSNorm(Norm):
+    """spec: size, eps.  Tensor: `<prefix>weight` [size]."""
+
+    def __init__(self, spec: PartSpec, dtype, device):
+        super().__init__(spec, dtype, device)
+        self.size = int(spec["size"])
+        self.eps = float(spec["eps"])
+        self.weight = None
+
+    @classmethod
+    def tensor_specs(cls, spec, prefix):
+        return [TensorSpec(prefix + "weight", (int(spec["size"]),), init="norm")]
+
+    def load(self, weights, prefix):
+        self.weight = weights[prefix + "weight"].contiguous()
+
+    def forward(self, residual):
+        return ops.add_rmsnorm(residual, None, self.weight, self.eps, self.dtype)
+
+    def add_forward(self, residual, delta, rows=None):
+        product = as_product(delta) if delta is not None else None
+        return ops.add_rmsnorm(residual, product, self.weight, self.eps, self.dtype, rows=rows)

@@ -1,0 +1,61 @@
+"""Random weights: writes a model folder (config.json, model.safetensors) from a configuration
+and a seed.  The reference has no such mode (every model-level test of it needs the real
+checkpoint); the list of tensors comes from the parts the model is built of, so a model with
+other parts gets other tensors without a change here.
+
+Each tensor is drawn from a generator seeded by (seed, tensor name): its values do not depend on
+which other tensors exist or in which order they are drawn.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+
+import torch
+
+from ..config.spec import TensorSpec
+from .safetensors_io import write_safetensors
+
+
+def _generator(seed: int, name: str) -> torch.Generator:
+    digest = hashlib.sha256(f"{seed}:{name}".encode("utf-8")).digest()
+    generator = torch.Generator(device="cpu")
+    generator.manual_seed(int.from_bytes(digest[:8], "little") & 0x7FFF_FFFF_FFFF_FFFF)
+    return generator
+
+
+def random_tensors(specs: list[TensorSpec], seed: int, std: float = 0.02, norm_std: float = 0.01,
+                   dtype: torch.dtype = torch.bfloat16) -> dict[str, torch.Tensor]:
+    out = {}
+    for spec in specs:
+        if spec.optional:
+            continue
+        generator = _generator(seed, spec.name)
+        values = torch.randn(spec.shape, generator=generator, dtype=torch.float32)
+        if spec.init == "normal":
+            values = values * std
+        elif spec.init == "norm":
+            values = 1.0 + values * norm_std
+        elif spec.init == "zeros":
+            values = torch.zeros(spec.shape)
+        else:
+            raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
+        out[spec.name] = values.to(dtype)
+    return out
+
+
+def write_random_model(model_dir: str, config, seed: int, std: float = 0.02, norm_std: float = 0.01,
+                       dtype: torch.dtype = torch.bfloat16) -> None:
+    """`config` is a configuration object of a registered architecture (it has `to_dict` and
+    `to_spec`).  The folder is created if needed."""
+    from ..models.builder import expected_tensors
+    os.makedirs(model_dir, exist_ok=True)
+    specs = expected_tensors(config.to_spec())
+    raw = config.to_dict()
+    raw["torch_dtype"] = {torch.bfloat16: "bfloat16", torch.float32: "float32", torch.float16: "float16"}[dtype]
+    with open(os.path.join(model_dir, "config.json"), "w", encoding="utf-8") as handle:
+        json.dump(raw, handle, indent=2, sort_keys=True)
+    write_safetensors(os.path.join(model_dir, "model.safetensors"),
+                      random_tensors(specs, seed, std, norm_std, dtype),
+                      metadata={"format": "pt", "seed": str(seed)})

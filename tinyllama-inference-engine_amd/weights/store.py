@@ -1,0 +1,113 @@
+"""Weights by tensor name, checked against what the model's parts expect.
+
+The reference's store answers `Get(name)` and `Validate(specs)`: every expected name present,
+with the expected shape, and no tensor beyond the expected ones (src/weight_store.cpp:264-295).
+It reports the first fault; here one error lists all of them: missing tensors, unexpected ones
+and wrong shapes.  Its code is `invalid_shape`, as the reference's is for each of the three.
+
+Kept precision: a tensor stored in 16-bit floating point is kept in bfloat16, a tensor stored in
+32-bit stays in 32-bit, integer tables become int32.  In the 32-bit mode every floating tensor is
+widened to float32.
+"""
+from __future__ import annotations
+
+import json
+import os
+import re
+from typing import Iterable
+
+import torch
+
+from ..config.spec import TensorSpec
+from ..errors import EngineError, ErrorCode
+from .safetensors_io import SafetensorsFile
+
+# buffers that some writers store although they are no weights
+_IGNORED = (re.compile(r".*\.rotary_emb\.inv_freq$"),)
+
+
+class WeightStore:
+    """All safetensors files of a model folder behind one `get(name)`."""
+
+    def __init__(self, model_dir: str):
+        self.model_dir = model_dir
+        self._files: list[SafetensorsFile] = []
+        self._where: dict[str, SafetensorsFile] = {}
+        index_path = os.path.join(model_dir, "model.safetensors.index.json")
+        single = os.path.join(model_dir, "model.safetensors")
+        if os.path.isfile(index_path):
+            try:
+                with open(index_path, "r", encoding="utf-8") as handle:
+                    weight_map = json.load(handle)["weight_map"]
+                names = sorted(set(weight_map.values()))
+            except (OSError, ValueError, KeyError, AttributeError) as error:
+                raise EngineError(ErrorCode.INVALID_FORMAT, f"{index_path}: not a shard index ({error})") from None
+        elif os.path.isfile(single):
+            names = ["model.safetensors"]
+        else:
+            raise EngineError(ErrorCode.IO, f"unable to open weights: {single} does not exist")
+        for name in names:
+            file = SafetensorsFile(os.path.join(model_dir, name))
+            self._files.append(file)
+            for tensor_name in file.tensors:
+                if tensor_name in self._where:
+                    raise EngineError(ErrorCode.INVALID_FORMAT, f"tensor '{tensor_name}' is stored in two files")
+                self._where[tensor_name] = file
+
+    def names(self) -> list[str]:
+        return sorted(self._where)
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._where
+
+    def shape(self, name: str) -> tuple[int, ...]:
+        return self._where[name].tensors[name].shape
+
+    def get(self, name: str) -> torch.Tensor:
+        if name not in self._where:
+            raise EngineError(ErrorCode.INVALID_SHAPE, f"required tensor is missing: {name}")
+        return self._where[name].tensor(name)
+
+    def validate(self, specs: Iterable[TensorSpec]) -> None:
+        specs = list(specs)
+        expected = {spec.name: spec for spec in specs}
+        missing = [spec.name for spec in specs if not spec.optional and spec.name not in self._where]
+        unexpected = [name for name in self.names()
+                      if name not in expected and not any(pattern.match(name) for pattern in _IGNORED)]
+        wrong = []
+        for spec in specs:
+            if spec.name in self._where and tuple(self.shape(spec.name)) != tuple(spec.shape):
+                wrong.append(f"{spec.name}: stored {list(self.shape(spec.name))}, expected {list(spec.shape)}")
+        if missing or unexpected or wrong:
+            parts = []
+            if missing:
+                parts.append(f"{len(missing)} missing: " + ", ".join(missing))
+            if unexpected:
+                parts.append(f"{len(unexpected)} unexpected: " + ", ".join(unexpected))
+            if wrong:
+                parts.append(f"{len(wrong)} with a wrong shape: " + "; ".join(wrong))
+            raise EngineError(ErrorCode.INVALID_SHAPE,
+                              f"weights in {self.model_dir} do not fit the model — " + " | ".join(parts))
+
+    def load(self, specs: Iterable[TensorSpec], dtype: torch.dtype, device) -> dict[str, torch.Tensor]:
+        """Validates, then uploads every expected tensor that is present, in its kept precision."""
+        specs = list(specs)
+        self.validate(specs)
+        out = {}
+        for spec in specs:
+            if spec.name in self._where:
+                out[spec.name] = to_kept_precision(self.get(spec.name), dtype).to(device)
+        return out
+
+
+def to_kept_precision(tensor: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """The precision a stored tensor is kept in when the model runs in `dtype`."""
+    if tensor.dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool):
+        return tensor.to(torch.int32)
+    if dtype == torch.float32:
+        return tensor.to(torch.float32)
+    if dtype == torch.bfloat16:
+        if tensor.dtype in (torch.float32, torch.float64):
+            return tensor.to(torch.float32)
+        return tensor.to(torch.bfloat16)
+    raise EngineError(ErrorCode.INVALID_DTYPE, f"the engine runs in bfloat16 or float32, not {dtype}")
