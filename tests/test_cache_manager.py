@@ -1,0 +1,168 @@
+"""The cache manager on the CPU: pages, block tables, groups, windows, request slots.
+
+The allocator's cases follow the reference's slot allocator (app/server.cpp:96-128: acquire until
+empty, release refuses what is not in use) and its cache tests (tests/unit_tests.cpp:173-196:
+out-of-range and budget errors), at page granularity."""
+import random
+
+import pytest
+import torch
+
+from tlie_amd import EngineError, ErrorCode
+from tlie_amd.cache import ABSENT, CacheManager, PageAllocator, RunNeed
+from tlie_amd.parts import KVCacheNeed, StateNeed
+
+
+def test_allocator_fifo_all_or_nothing_and_double_free():
+    pool = PageAllocator(4)
+    assert pool.alloc(3) == [0, 1, 2] and pool.num_free == 1
+    assert pool.alloc(2) is None and pool.num_free == 1          # nothing taken
+    pool.release([1])
+    assert pool.alloc(2) == [3, 1]                                # FIFO: the returned page comes last
+    with pytest.raises(EngineError):
+        pool.release([7])
+    pool.release([0])
+    with pytest.raises(EngineError):
+        pool.release([0])                                         # freed twice
+    with pytest.raises(EngineError):
+        pool.release([2, 2])
+    assert pool.in_use(2) and pool.num_used == 3                  # a refused call frees nothing
+    with pytest.raises(EngineError):
+        PageAllocator(0)
+
+
+def manager(num_pages=8, page_size=4, max_requests=3, window=None, state=False, runs=2):
+    needs = [RunNeed(cache_of=i, kv=KVCacheNeed(2, 8, window), state=StateNeed((5,)) if state else None) for i in range(runs)]
+    return CacheManager(needs, page_size, num_pages, max_requests, torch.float32, "cpu", max_positions=64)
+
+
+def test_pages_follow_length_and_come_back():
+    cache = manager()
+    assert cache.admit("a") == 0 and cache.admit("b") == 1
+    assert cache.pages_needed("a", 5) == [2]
+    cache.reserve("a", 5)
+    assert cache.page_list("a", 0) == [0, 1] and cache.length("a") == 0
+    assert cache.rows("a", 0, 3, 2) == [3, 4]                     # position 3 on page 0, position 4 on page 1 row 0
+    cache.commit("a", 5)
+    assert cache.length("a") == 5 and cache.pages_needed("a", 3) == [0] and cache.pages_needed("a", 4) == [1]
+    cache.reserve("b", 9)
+    cache.commit("b", 9)
+    assert cache.page_list("b", 0) == [2, 3, 4] and cache.free_pages() == [3]
+    assert cache.can_reserve([("a", 3), ("b", 8)]) and not cache.can_reserve([("a", 4), ("b", 12)])
+    with pytest.raises(EngineError) as caught:
+        cache.reserve("b", 16)
+    assert caught.value.code == ErrorCode.OUT_OF_MEMORY and cache.page_list("b", 0) == [2, 3, 4]
+    cache.release("a")
+    cache.check()
+    assert cache.free_pages() == [5]
+    cache.admit("c")                                              # the slot of "a" is used again
+    assert cache.slot("c") == 0
+    cache.reserve("c", 16)
+    assert cache.page_list("c", 0) == [5, 6, 7, 0]                # FIFO: the pages "a" gave back come last
+    cache.check()
+    with pytest.raises(EngineError):
+        cache.commit("c", 17)                                     # more than was reserved
+    with pytest.raises(EngineError):
+        cache.admit("c")
+    with pytest.raises(EngineError):
+        cache.length("nobody")
+    with pytest.raises(EngineError) as caught:
+        cache.reserve("c", 65)
+    assert caught.value.code == ErrorCode.OUT_OF_BOUNDS           # past the model's positions
+
+
+def test_request_slots_run_out_and_state_starts_at_zero():
+    cache = manager(max_requests=2, state=True)
+    assert len(cache.state_areas) == 2 and cache.state_areas[0].shape == (2, 5)
+    cache.admit("a")
+    cache.admit("b")
+    with pytest.raises(EngineError) as caught:
+        cache.admit("c")
+    assert caught.value.code == ErrorCode.OUT_OF_MEMORY
+    cache.bindings[0].state[cache.slot("b")] += 3.0
+    cache.release("b")
+    assert cache.admit("c") == 1 and float(cache.bindings[0].state[1].abs().sum()) == 0.0
+    assert cache.bindings[0].state is not cache.bindings[1].state
+
+
+def test_groups_by_need_and_shared_caches():
+    needs = [RunNeed(0, KVCacheNeed(2, 8, None)), RunNeed(1, KVCacheNeed(1, 16, 6)), RunNeed(0, KVCacheNeed(2, 8, None)),
+             RunNeed(3, None), RunNeed(4, KVCacheNeed(2, 8, 6))]
+    cache = CacheManager(needs, 4, 6, 2, torch.float32, "cpu")
+    assert [group.window for group in cache.groups] == [None, 6]
+    assert [b.group for b in cache.bindings] == [0, 1, 0, None, 1]
+    assert cache.bindings[2].cache is cache.bindings[0].cache and not cache.bindings[2].writes and cache.bindings[0].writes
+    assert cache.bindings[1].cache.shape == (6, 2, 1, 4, 16) and cache.bindings[4].cache.shape == (6, 2, 2, 4, 8)
+    with pytest.raises(EngineError):
+        CacheManager([RunNeed(0, KVCacheNeed(2, 8)), RunNeed(0, KVCacheNeed(1, 8))], 4, 6, 2, torch.float32, "cpu")
+    # the windowed group gives pages back as the request grows; the full group keeps them
+    cache.admit("a")
+    for _ in range(5):
+        cache.reserve("a", 4)
+        cache.commit("a", 4)
+        cache.check()
+    assert cache.length("a") == 20
+    assert cache.page_list("a", 0) == [0, 1, 2, 3, 4]
+    # window 6 at length 20: a later token (position >= 20) sees keys >= 15, so blocks 0..2 (positions 0..11) are gone
+    assert [page == ABSENT for page in cache.page_list("a", 1)] == [True, True, True, False, False]
+    assert cache.free_pages() == [1, 4]
+    with pytest.raises(EngineError):
+        cache.rows("a", 1, 11, 1)
+    assert len(cache.rows("a", 1, 12, 8)) == 8
+    cache.release("a")
+    cache.check()
+    assert cache.free_pages() == [6, 6]
+
+
+def test_window_edge_exactly():
+    cache = manager(num_pages=8, page_size=4, window=4, runs=1)
+    cache.admit("a")
+    cache.reserve("a", 7)
+    cache.commit("a", 7)       # next position 7 sees keys 4..7: block 0 (0..3) is dead
+    assert [p == ABSENT for p in cache.page_list("a", 0)] == [True, False]
+    cache.reserve("a", 1)
+    cache.commit("a", 1)       # length 8: position 8 sees 5..8, block 1 still holds 5, 6, 7
+    assert [p == ABSENT for p in cache.page_list("a", 0)] == [True, False]
+    cache.reserve("a", 3)
+    cache.commit("a", 3)       # length 11: position 11 sees 8..11, block 1 (4..7) is dead
+    assert [p == ABSENT for p in cache.page_list("a", 0)] == [True, True, False]
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_lose_nothing(seed):
+    rng = random.Random(seed)
+    window = [None, 5, None, 9, 3, None][seed]
+    cache = manager(num_pages=12, page_size=4, max_requests=4, window=window, runs=2)
+    live, counter = [], 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.25 and cache.free_slots > 0:
+            counter += 1
+            cache.admit(counter)
+            live.append(counter)
+        elif action < 0.8 and live:
+            request = rng.choice(live)
+            count = rng.randint(1, 9)
+            if cache.length(request) + count > 64:
+                continue
+            if cache.can_reserve([(request, count)]):
+                cache.reserve(request, count)
+                rows = cache.rows(request, 0, cache.length(request), count)
+                assert len(set(rows)) == count
+                cache.commit(request, count)
+            else:
+                with pytest.raises(EngineError):
+                    cache.reserve(request, count)
+        elif live:
+            request = live.pop(rng.randrange(len(live)))
+            cache.release(request)
+            with pytest.raises(EngineError):
+                cache.release(request)
+        cache.check()
+        # no row of the cache belongs to two live requests
+        held = [page for request in live for page in cache.page_list(request, 0) if page != ABSENT]
+        assert len(held) == len(set(held))
+    for request in live:
+        cache.release(request)
+    cache.check()
+    assert cache.free_pages() == [12] and cache.free_slots == 4

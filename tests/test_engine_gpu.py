@@ -1,0 +1,254 @@
+"""The engine on the GPU against the plain implementation: every way of cutting the work, in
+32-bit and in bfloat16, for both tiny configurations."""
+import json
+import os
+import random
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from gpu_helpers import (CONFIGS, CUT_TOLERANCE, DTYPES, TOLERANCE, Replayer, assert_close, first_bad_row, load_plain,
+                         make_model, random_tokens)
+from plain_llama import plain_forward, plain_generate_greedy
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CASES = [(name, dtype) for name in CONFIGS for dtype in DTYPES]
+
+
+@pytest.fixture(scope="module")
+def setups(tmp_path_factory):
+    """Per (configuration, dtype): model folder, plain config and weights, and a cache of plain logits."""
+    made = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in made:
+            folder = make_model(tmp_path_factory.mktemp(f"model_{name}_{dtype}"), CONFIGS[name], seed=11, dtype_name=dtype)
+            raw, weights = load_plain(folder)
+            made[(name, dtype)] = {"folder": folder, "raw": raw, "weights": weights, "plain": {}}
+        return made[(name, dtype)]
+    return get
+
+
+def plain_logits(setup, tokens):
+    key = tuple(tokens)
+    if key not in setup["plain"]:
+        setup["plain"][key] = plain_forward(setup["raw"], setup["weights"], list(tokens))
+    return setup["plain"][key]
+
+
+def new_engine(setup, dtype, max_tokens=512, page_size=16, max_requests=4):
+    from tlie_amd import Engine
+    return Engine(setup["folder"], dtype=dtype, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests)
+
+
+def request_tokens(name, index, length):
+    return random_tokens(1000 * index + length, length, CONFIGS[name]["vocab_size"])
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_whole_and_alone(setups, name, dtype):
+    setup = setups(name, dtype)
+    engine = new_engine(setup, dtype)
+    for index, length in enumerate((1, 2, 17, 100 if name == "A" else 150)):
+        tokens = request_tokens(name, index, length)
+        replay = Replayer(engine)
+        replay.step([("r", tokens, list(range(length)))], end=["r"])
+        got = replay.logits_of("r", range(length))
+        want = plain_logits(setup, tokens)
+        bad = first_bad_row(got, want, TOLERANCE[dtype])
+        assert bad is None, f"{name} {dtype} length {length}: first wrong position {bad}"
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_most_in_one_step_then_the_last_32_one_by_one(setups, name, dtype):
+    setup = setups(name, dtype)
+    engine = new_engine(setup, dtype)
+    length = 90 if name == "A" else 131
+    tokens = request_tokens(name, 7, length)
+    whole = Replayer(engine)
+    whole.step([("w", tokens, list(range(length)))], end=["w"])
+    cut = Replayer(engine)
+    cut.step([("c", tokens[:length - 32], list(range(length - 32)))])
+    for position in range(length - 32, length):
+        cut.step([("c", [tokens[position]], [0])])
+    engine.finish("c")
+    got = cut.logits_of("c", range(length))
+    assert first_bad_row(got, plain_logits(setup, tokens), TOLERANCE[dtype]) is None
+    bad = first_bad_row(got, whole.logits_of("w", range(length)), CUT_TOLERANCE[dtype])
+    assert bad is None, f"decoded position {bad} differs from the whole prompt's"
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_portions_of_changing_size(setups, name, dtype):
+    setup = setups(name, dtype)
+    engine = new_engine(setup, dtype)
+    length = 101 if name == "A" else 160
+    tokens = request_tokens(name, 3, length)
+    sizes = [16, 7, 2, 5, 3, 2, 1, 17, 2, 31, 2, 2, 1, 1, 9]
+    replay = Replayer(engine)
+    cursor, turn = 0, 0
+    while cursor < length:
+        size = min(sizes[turn % len(sizes)], length - cursor)
+        replay.step([("p", tokens[cursor:cursor + size], list(range(size)))])
+        cursor += size
+        turn += 1
+    engine.finish("p")
+    got = replay.logits_of("p", range(length))
+    bad = first_bad_row(got, plain_logits(setup, tokens), TOLERANCE[dtype])
+    assert bad is None, f"first wrong position {bad} (page size 16; portions {sizes})"
+
+
+def mixed_trace(name, seed, requests=7, live_limit=4):
+    """A seeded trace: up to four live requests, portions of some beside single decoded tokens of
+    others, requests ending and new ones starting mid-trace.  Returns (steps, token lists, the
+    most 64-rounded positions live at once)."""
+    rng = random.Random(seed)
+    limit = CONFIGS[name]["max_position_embeddings"]
+    lengths = [rng.randint(34, min(limit, 120)) for _ in range(requests)]
+    tokens = {f"r{i}": request_tokens(name, 50 + i, lengths[i]) for i in range(requests)}
+    waiting = list(tokens)
+    live, done_at, steps, most = {}, {}, [], 0
+    while waiting or live:
+        while waiting and len(live) < live_limit and (not live or rng.random() < 0.6):
+            live[waiting.pop(0)] = 0
+        items, ending = [], []
+        for request in list(live):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                                   # left out of this step, goes on later
+            at, total = live[request], len(tokens[request])
+            decode_from = total - 12
+            size = 1 if at >= decode_from else min(rng.choice([2, 3, 5, 8, 16, 23]), decode_from - at)
+            items.append((request, tokens[request][at:at + size], list(range(size))))
+            live[request] = at + size
+            if live[request] == total:
+                ending.append(request)
+        most = max(most, sum(-(-max(at, 1) // 64) * 64 for at in live.values()))
+        if items:
+            steps.append((items, ending))
+        for request in ending:
+            del live[request]
+    return steps, tokens, most
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_mixed_requests_with_pages_used_again(setups, name, dtype):
+    setup = setups(name, dtype)
+    steps, tokens, most = mixed_trace(name, seed=5)
+    engine = new_engine(setup, dtype, max_tokens=most, page_size=16, max_requests=4)
+    pages_seen = {}
+    replay = Replayer(engine)
+    for items, ending in steps:
+        replay.step(items, end=())
+        for request, _, _ in items:
+            pages_seen.setdefault(request, set()).update(engine.cache.page_list(request, 0))
+        for request in ending:
+            engine.finish(request)
+    owners = {}
+    for request, pages in pages_seen.items():
+        for page in pages:
+            owners.setdefault(page, set()).add(request)
+    assert any(len(users) > 1 for users in owners.values()), "the trace never used a page again"
+    for request, sequence in tokens.items():
+        got = replay.logits_of(request, range(len(sequence)))
+        bad = first_bad_row(got, plain_logits(setup, sequence), TOLERANCE[dtype])
+        assert bad is None, f"{request}: first wrong position {bad} of {len(sequence)}"
+    assert engine.cache.free_pages() == [engine.cache.num_pages] and engine.cache.free_slots == 4
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_long_decoding_and_first_tokens(setups, name, dtype):
+    setup = setups(name, dtype)
+    engine = new_engine(setup, dtype)
+    length = CONFIGS[name]["max_position_embeddings"]
+    tokens = request_tokens(name, 9, length)
+    replay = Replayer(engine)
+    for position in range(length):                      # every token of the sequence decoded one by one, from the first
+        replay.step([("d", [tokens[position]], [0])])
+    engine.finish("d")
+    got = replay.logits_of("d", range(length))
+    want = plain_logits(setup, tokens)
+    assert_close(got[:4], want[:4], TOLERANCE[dtype], "the first tokens of a sequence")
+    bad = first_bad_row(got, want, TOLERANCE[dtype])
+    assert bad is None, f"first wrong position {bad} of {length}"
+    from tlie_amd import EngineError, StepEntry
+    engine.admit("over")
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("over", tokens + [1], [])])          # past the model's positions
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("over", [CONFIGS[name]["vocab_size"]], [0])])   # token outside the vocabulary
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("over", [1], [0]), StepEntry("over", [2], [0])])  # a request twice in a step
+    engine.finish("over")
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_greedy_generation_through_the_entry_point(setups, name, dtype):
+    setup = setups(name, dtype)
+    engine = new_engine(setup, dtype)
+    prompts = [request_tokens(name, 20 + i, n) for i, n in enumerate((16, 5, 37))]
+    got = engine.generate(prompts, max_tokens=16, chunk_size=16, max_tokens_per_step=24)
+    for prompt, tokens in zip(prompts, got):
+        want = plain_generate_greedy(setup["raw"], setup["weights"], prompt, 16)
+        if dtype == "float32":
+            assert tokens == want
+        else:
+            # bfloat16 may pick another token where the two best logits are closer than its rounding;
+            # up to the first such place the tokens are the same, and that place must be a near tie
+            same = next((i for i, (a, b) in enumerate(zip(tokens, want)) if a != b), len(want))
+            if same < len(want):
+                logits = plain_forward(setup["raw"], setup["weights"], prompt + want[:same])[-1]
+                gap = (logits[want[same]] - logits[tokens[same]]).item()
+                assert 0 <= gap <= 2 * TOLERANCE[dtype] * logits.abs().max().item(), f"token {same} differs without a near tie"
+    assert engine.cache.free_pages() == [engine.cache.num_pages]
+
+
+def error_code(stderr):
+    """The error line is the last line of standard error (the GPU's driver may print before it)."""
+    return json.loads(stderr.strip().splitlines()[-1])["error"]["code"]
+
+
+def test_replay_program_and_command_line(setups, tmp_path):
+    """bin/trace_run and bin/tinyllama_amd as a user runs them: separate processes."""
+    setup = setups("A", "float32")
+    tokens = request_tokens("A", 1, 40)
+    other = request_tokens("A", 2, 21)
+    lines = [
+        {"step": 0, "entries": [{"id": "a", "tokens": tokens[:30], "want": [0, 29]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": tokens[30:32], "want": []}, {"id": "b", "tokens": other, "want": [20]}], "end": ["b"]},
+        {"step": 2, "entries": [{"id": "a", "tokens": tokens[32:], "want": [7]}], "end": ["a"]},
+    ]
+    out = tmp_path / "logits"
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", setup["folder"], "--dtype", "float32",
+                          "--out", str(out), "--max-tokens", "128"], input="\n".join(json.dumps(line) for line in lines) + "\n",
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert run.stdout.split() == ["done", "0", "done", "1", "done", "2"]
+    import numpy
+    vocab = CONFIGS["A"]["vocab_size"]
+    step0 = torch.from_numpy(numpy.fromfile(out / "0.f32", dtype="<f4").reshape(-1, vocab))
+    step1 = torch.from_numpy(numpy.fromfile(out / "1.f32", dtype="<f4").reshape(-1, vocab))
+    step2 = torch.from_numpy(numpy.fromfile(out / "2.f32", dtype="<f4").reshape(-1, vocab))
+    want = plain_logits(setup, tokens)
+    assert_close(step0, want[[0, 29]], TOLERANCE["float32"], "step 0")
+    assert_close(step1, plain_logits(setup, other)[[20]], TOLERANCE["float32"], "step 1")
+    assert_close(step2, want[[39]], TOLERANCE["float32"], "step 2")
+
+    prompt = "ids:" + ",".join(str(token) for token in tokens[:9])
+    cli = [sys.executable, os.path.join(ROOT, "bin", "tinyllama_amd")]
+    run = subprocess.run(cli + ["generate", setup["folder"], prompt, "6", "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    result = json.loads(run.stdout)
+    assert result["prompt_tokens"] == 9
+    assert result["generated_tokens"] == plain_generate_greedy(setup["raw"], setup["weights"], tokens[:9], 6)
+    run = subprocess.run(cli + ["logits", setup["folder"], prompt, "--dtype", "float32"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr
+    assert_close(torch.tensor(json.loads(run.stdout)["logits"]), plain_logits(setup, tokens[:9])[-1], TOLERANCE["float32"], "logits")
+    run = subprocess.run(cli + ["generate", setup["folder"], prompt, "many"], capture_output=True, text=True, timeout=300)
+    assert run.returncode != 0 and error_code(run.stderr) == "invalid_argument"     # tests/expect_cli_failure.cmake
+    run = subprocess.run(cli + ["generate", setup["folder"], "some text", "4"], capture_output=True, text=True, timeout=300)
+    assert run.returncode != 0 and error_code(run.stderr) == "tokenizer_error"
+    run = subprocess.run(cli + ["generate", setup["folder"], prompt, "200"], capture_output=True, text=True, timeout=300)
+    assert run.returncode != 0 and error_code(run.stderr) == "out_of_bounds"         # app/reference_cli.cpp:72-75

@@ -1,0 +1,270 @@
+"""Each HIP kernel alone against its plain reference, at sizes other than the engine's tiny
+configurations (no power of two, odd head counts), in float32 and bfloat16, and with inputs built
+so that a fault at a special place shows: a far key among hundreds, a page's edge, a window's edge,
+pages in shuffled physical order."""
+import math
+import random
+
+import pytest
+import torch
+
+from plain_llama import (plain_attention, plain_greedy, plain_linear, plain_rms_norm, plain_rope, plain_silu_mul,
+                         plain_top_p_distribution)
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 2e-6, "bfloat16": 1.2e-2}      # relative to the largest expected value; bf16 = 2^-8 output rounding + input rounding
+
+
+def rel_err(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return ((got - want).abs().max() / want.abs().max().clamp_min(1e-30)).item()
+
+
+def rounded(tensor, dtype):
+    """The values a kernel sees: rounded to the storage type, as float64 for the plain reference."""
+    return tensor.to(dtype).double()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_embed_gather(dtype):
+    from tlie_amd import ops
+    table = torch.randn(301, 72).to(DT[dtype]).to(DEV)
+    tokens = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
+    out = ops.embed_gather(tokens, table)
+    assert out.dtype == torch.float32 and torch.equal(out.cpu(), table.float().cpu()[tokens.long().cpu()])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("hidden", [72, 1000, 2048, 5000])
+def test_add_rmsnorm(dtype, hidden):
+    from tlie_amd import ops
+    torch.manual_seed(hidden)
+    tokens = 7
+    residual = torch.randn(tokens, hidden) * 3
+    delta = (torch.randn(3, tokens, hidden)).float()
+    weight = (1 + 0.2 * torch.randn(hidden)).to(DT[dtype])
+    eps = 1e-6
+    res_dev = residual.to(DEV)
+    out = ops.add_rmsnorm(res_dev, ops.Product(delta.to(DEV), 3), weight.to(DEV), eps, DT[dtype])
+    summed = residual.double() + delta.double().sum(0)
+    assert rel_err(res_dev, summed) < 2e-6                                  # the residual sum is 32-bit in both modes
+    assert rel_err(out, plain_rms_norm(summed, weight.double(), eps)) < TOL[dtype]
+    # norm only, golden vector of the reference (data/golden/operators.json:4-24)
+    x = torch.tensor([[1.0, -2.0, 3.0, -4.0]], device=DEV)
+    w = torch.tensor([0.5, 1.0, 1.5, 2.0], device=DEV)
+    got = ops.add_rmsnorm(x, None, w, 1e-5, torch.float32)
+    want = torch.tensor([[0.182574063539505, -0.73029625415802, 1.6431666612625122, -2.92118501663208]])
+    assert torch.allclose(got.cpu(), want, atol=1e-6, rtol=0)
+    # picked rows: the residual is left alone, the output is norm(residual + delta) of those rows
+    res_dev = residual.to(DEV)
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32, device=DEV)
+    one = ops.Product(delta[0].to(DT[dtype]).to(DEV).contiguous(), 1)
+    picked = ops.add_rmsnorm(res_dev, one, weight.to(DEV), eps, DT[dtype], rows=rows)
+    assert torch.equal(res_dev.cpu(), residual)
+    want = plain_rms_norm(residual.double()[[5, 0, 5]] + rounded(delta[0], DT[dtype])[[5, 0, 5]], weight.double(), eps)
+    assert rel_err(picked, want) < TOL[dtype]
+    # a zero row gives zero, not NaN (eps is inside the root)
+    zero = ops.add_rmsnorm(torch.zeros(1, hidden, device=DEV), None, weight.to(DEV), eps, DT[dtype])
+    assert float(zero.float().abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_silu_mul(dtype):
+    from tlie_amd import ops
+    gate_up = torch.tensor([[-2.0, -0.5, 0.0, 1.5, 0.5, -1.0, 2.0, 3.0]], device=DEV)      # operators.json:132-151
+    got = ops.silu_mul(ops.Product(gate_up, 1), torch.float32)
+    want = torch.tensor([[-0.11920291930437088, 0.1887703388929367, 0.0, 3.6790847778320312]])
+    assert torch.allclose(got.cpu(), want, atol=1e-6, rtol=0)
+    torch.manual_seed(0)
+    parts = torch.randn(2, 9, 2 * 177) * 2
+    got = ops.silu_mul(ops.Product(parts.to(DEV), 2), DT[dtype])
+    total = parts.double().sum(0)
+    assert rel_err(got, plain_silu_mul(total[:, :177], total[:, 177:])) < TOL[dtype]
+    extreme = torch.tensor([[80.0, -90.0, 2.0, 2.0]], device=DEV)
+    got = ops.silu_mul(ops.Product(extreme, 1), torch.float32).cpu()
+    assert got[0, 0] == 160.0 and abs(got[0, 1]) < 1e-30 and torch.isfinite(got).all()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(1, 40, 24), (5, 72, 100), (70, 129, 333), (130, 64, 2048)])
+def test_gemm_generic(dtype, shape):
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(m)
+    x = torch.randn(m, k).to(DT[dtype])
+    w = (torch.randn(n, k) / math.sqrt(k)).to(DT[dtype])
+    b = torch.randn(n).to(DT[dtype])
+    got = ops.gemm_generic(x.to(DEV), w.to(DEV), b.to(DEV), torch.float32).dense()
+    assert rel_err(got, plain_linear(x.double(), w.double(), b.double())) < 5e-6
+    got = ops.gemm_generic(x.to(DEV), w.to(DEV), None, DT[dtype]).dense()
+    assert rel_err(got, plain_linear(x.double(), w.double())) < TOL[dtype]
+
+
+def test_gemm_is_true_32_bit():
+    """(1 + 2^-12)^2 accumulated onto -(1 + 2^-11) leaves 2^-24: it needs all 24 bits of both
+    factors and a fused multiply-add; a product whose inputs were cut to fewer bits leaves -2^-11
+    or 0.  (The sum runs in index order, so the negative term is accumulated first.)"""
+    from tlie_amd import ops
+    a = 1.0 + 2.0 ** -12
+    x = torch.tensor([[1.0, a] + [0.0] * 30], device=DEV)
+    w = torch.tensor([[-(1.0 + 2.0 ** -11), a] + [0.0] * 30], device=DEV)
+    got = ops.gemm_generic(x, w, None, torch.float32).dense().item()
+    assert got == 2.0 ** -24
+
+
+def build_cache(k, v, page_size, dtype, shuffle_seed=0, extra_pages=3):
+    """Puts one sequence's keys and values [T, nkv, d] on pages in shuffled physical order.
+    Returns (cache [pages, 2, nkv, page_size, d], block table row)."""
+    tokens, nkv, d = k.shape
+    blocks = (tokens + page_size - 1) // page_size
+    order = list(range(blocks + extra_pages))
+    random.Random(shuffle_seed).shuffle(order)
+    cache = torch.full((blocks + extra_pages, 2, nkv, page_size, d), 7.5).to(dtype)     # stale rows hold a loud value
+    for position in range(tokens):
+        page, row = order[position // page_size], position % page_size
+        cache[page, 0, :, row] = k[position].to(dtype)
+        cache[page, 1, :, row] = v[position].to(dtype)
+    return cache, order[:blocks]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", [
+    dict(tokens=3, nq=2, nkv=1, d=4, page=16, golden=True),
+    dict(tokens=77, nq=6, nkv=3, d=48, page=16),
+    dict(tokens=300, nq=5, nkv=5, d=80, page=32),
+    dict(tokens=700, nq=8, nkv=1, d=128, page=16, window=None),
+    dict(tokens=333, nq=4, nkv=2, d=16, page=8, window=37),
+    dict(tokens=130, nq=3, nkv=1, d=256, page=64),
+])
+def test_attention_generic(dtype, case):
+    from tlie_amd import ops
+    tokens, nq, nkv, d, page = case["tokens"], case["nq"], case["nkv"], case["d"], case["page"]
+    window = case.get("window")
+    torch.manual_seed(tokens)
+    if case.get("golden"):                                               # data/golden/operators.json:78-131
+        q = torch.zeros(3, 2, 4)
+        q[2] = torch.tensor([0.2, -0.1, 0.4, 0.3, -0.5, 0.7, 0.1, -0.2]).view(2, 4)
+        k = torch.tensor([0.1, 0.2, 0.3, 0.4, -0.4, 0.3, -0.2, 0.1, 0.5, -0.6, 0.7, -0.8]).view(3, 1, 4)
+        v = torch.tensor([1.0, 0.0, -1.0, 0.5, 0.2, 0.4, 0.6, 0.8, -0.3, 0.7, 0.9, -0.1]).view(3, 1, 4)
+    else:
+        q, k, v = torch.randn(tokens, nq, d), torch.randn(tokens, nkv, d), torch.randn(tokens, nkv, d)
+    cache, pages = build_cache(k, v, page, DT[dtype], shuffle_seed=tokens)
+    table = torch.tensor([[0] * len(pages), pages], dtype=torch.int32, device=DEV)      # row 1 is the sequence
+    token_seq = torch.ones(tokens, dtype=torch.int32, device=DEV)
+    positions = torch.arange(tokens, dtype=torch.int32, device=DEV)
+    got = ops.attention_generic(q.to(DT[dtype]).view(tokens, nq * d).to(DEV), cache.to(DEV), table, token_seq, positions,
+                                nq, nkv, d, window, 1.0 / math.sqrt(d)).view(tokens, nq, d)
+    want = plain_attention(rounded(q, DT[dtype]), rounded(k, DT[dtype]), rounded(v, DT[dtype]), window=window)
+    assert rel_err(got, want) < TOL[dtype]
+    if case.get("golden"):
+        golden = torch.tensor([0.31072109937667847, 0.3621496558189392, 0.13341431319713593, 0.3776317536830902,
+                               0.3371150493621826, 0.3447031080722809, 0.14012068510055542, 0.46016252040863037])
+        if dtype == "float32":
+            assert torch.allclose(got[2].flatten().cpu().double(), golden.double(), atol=1e-6, rtol=0)
+    # a step that brings only some of the tokens (a portion, or one decoded token) gives the same rows
+    some = [tokens - 1] if tokens < 5 else [0, 1, page - 1, page, page + 1, tokens // 2, tokens - 2, tokens - 1]
+    sub = ops.attention_generic(q[some].to(DT[dtype]).reshape(len(some), nq * d).to(DEV).contiguous(), cache.to(DEV), table,
+                                torch.ones(len(some), dtype=torch.int32, device=DEV),
+                                torch.tensor(some, dtype=torch.int32, device=DEV), nq, nkv, d, window, 1.0 / math.sqrt(d))
+    assert torch.equal(sub.view(len(some), nq, d).cpu(), got[some].cpu())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_attention_finds_one_key_among_hundreds(dtype):
+    """One key is made to stand out (its score is far above the rest), at places where an index
+    mistake would miss it: the first key, a page's last row and the next page's first, the last
+    key but one, the window's first key and the key just outside the window."""
+    from tlie_amd import ops
+    tokens, nq, nkv, d, page = 600, 4, 2, 32, 16
+    torch.manual_seed(1)
+    base_k, v = torch.randn(tokens, nkv, d) * 0.1, torch.randn(tokens, nkv, d)
+    q = torch.randn(1, nq, d) * 0.1
+    direction = torch.zeros(d)
+    direction[3] = 1.0
+    q = q + 12.0 * direction
+    position = tokens - 1
+    for window, needle, inside in [(None, 0, True), (None, 15, True), (None, 16, True), (None, 511, True), (None, 598, True),
+                                   (100, 500, True), (100, 499, False), (100, 599, True), (16, 584, True), (16, 583, False)]:
+        k = base_k.clone()
+        k[needle] += 12.0 * direction                   # score about 144 / sqrt(32) = 25 above the others
+        cache, pages = build_cache(k, v, page, DT[dtype], shuffle_seed=needle)
+        got = ops.attention_generic(q.to(DT[dtype]).view(1, nq * d).to(DEV), cache.to(DEV),
+                                    torch.tensor([pages], dtype=torch.int32, device=DEV),
+                                    torch.zeros(1, dtype=torch.int32, device=DEV),
+                                    torch.tensor([position], dtype=torch.int32, device=DEV), nq, nkv, d, window,
+                                    1.0 / math.sqrt(d)).view(nq, d).float().cpu()
+        wanted_rows = rounded(v[needle], DT[dtype]).float().repeat_interleave(nq // nkv, dim=0)
+        hit = (got - wanted_rows).abs().max().item() < 0.05
+        assert hit == inside, f"window {window}, needle at {needle}: {'missed' if inside else 'seen'}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rope_cache(dtype):
+    from tlie_amd import ops
+    # the reference's golden vector (data/golden/operators.json:25-63): 2 q heads, 1 kv head, d = 4, position 7
+    qkv = torch.tensor([[0.1, 0.2, 0.3, 0.4, -0.5, 0.6, -0.7, 0.8, 0.9, -1.0, 1.1, -1.2, 5.0, 6.0, 7.0, 8.0]], device=DEV)
+    inv_freq = torch.pow(torch.tensor(10000.0), -2.0 * torch.arange(2, dtype=torch.float32) / 4.0).to(DEV)
+    cache = torch.zeros(3, 2, 1, 4, 4, device=DEV)
+    q = ops.rope_cache(ops.Product(qkv, 1), torch.tensor([7], dtype=torch.int32, device=DEV),
+                       torch.tensor([2 * 4 + 1], dtype=torch.int32, device=DEV), inv_freq, 4, cache, 2, 1, 4, torch.float32)
+    want_q = torch.tensor([-0.12170576304197311, 0.17153306305408478, 0.2918693423271179, 0.41300898790359497,
+                           0.08293947577476501, 0.5425763726234436, -0.8562248945236206, 0.8400065302848816])
+    want_k = torch.tensor([-0.044173240661621094, -0.9136196374893188, 1.4205803871154785, -1.267004132270813])
+    assert torch.allclose(q.cpu().flatten(), want_q, atol=1e-6, rtol=0)
+    assert torch.allclose(cache[2, 0, 0, 1].cpu(), want_k, atol=1e-6, rtol=0)
+    assert torch.equal(cache[2, 1, 0, 1].cpu(), torch.tensor([5.0, 6.0, 7.0, 8.0]))      # the value is stored unrotated
+    assert float(cache.abs().sum()) == pytest.approx(float(want_k.abs().sum()) + 26.0, rel=1e-5)   # nothing else was written
+
+    # other sizes, split partial sums, far positions (the reference tests position 4095: tests/cuda/kernel_tests.cu:144-146)
+    tokens, nq, nkv, d, page = 9, 5, 3, 48, 8
+    torch.manual_seed(3)
+    parts = torch.randn(2, tokens, (nq + 2 * nkv) * d)
+    positions = torch.tensor([0, 1, 2, 4095, 77, 1000, 8, 9, 31], dtype=torch.int32)
+    slots = torch.tensor([3, 12, -1, 40, 41, 7, 0, 63, 20], dtype=torch.int32)
+    theta = 500000.0
+    inv_freq = torch.pow(torch.tensor(theta), -2.0 * torch.arange(d // 2, dtype=torch.float32) / d).to(DEV)
+    cache = torch.full((8, 2, nkv, page, d), -3.0).to(DT[dtype]).to(DEV)
+    q = ops.rope_cache(ops.Product(parts.to(DEV), 2), positions.to(DEV), slots.to(DEV), inv_freq, d, cache, nq, nkv, d, DT[dtype])
+    total = parts.double().sum(0)
+    want_q = plain_rope(total[:, :nq * d].view(tokens, nq, d), positions, theta)
+    want_k = plain_rope(total[:, nq * d:(nq + nkv) * d].view(tokens, nkv, d), positions, theta)
+    want_v = total[:, (nq + nkv) * d:].view(tokens, nkv, d)
+    assert rel_err(q.view(tokens, nq, d), want_q) < TOL[dtype]
+    cache = cache.cpu()
+    written = torch.zeros(8, page, dtype=torch.bool)
+    for t in range(tokens):
+        if slots[t] < 0:
+            continue
+        page_index, row = int(slots[t]) // page, int(slots[t]) % page
+        written[page_index, row] = True
+        assert rel_err(cache[page_index, 0, :, row], want_k[t]) < TOL[dtype]
+        assert rel_err(cache[page_index, 1, :, row], want_v[t]) < TOL[dtype]
+    for page_index in range(8):
+        for row in range(page):
+            if not written[page_index, row]:
+                assert float((cache[page_index, :, :, row].float() + 3.0).abs().max()) == 0.0
+    # no rotation table: q and k pass through
+    plain_q = ops.rope_cache(ops.Product(parts[0].to(DEV).contiguous(), 1), positions.to(DEV), slots.to(DEV), None, 0,
+                             torch.zeros(8, 2, nkv, page, d, dtype=DT[dtype], device=DEV), nq, nkv, d, DT[dtype])
+    assert rel_err(plain_q, parts[0][:, :nq * d]) < TOL[dtype]
+
+
+def test_kernels_refuse_what_they_do_not_take():
+    from tlie_amd import EngineError, ops
+    x = torch.randn(4, 8, device=DEV)
+    with pytest.raises(EngineError):
+        ops.gemm_generic(x, torch.randn(5, 9, device=DEV), None, torch.float32)                  # inner sizes differ
+    with pytest.raises(EngineError):
+        ops.gemm_generic(x.cpu(), torch.randn(5, 8), None, torch.float32)                        # not on the GPU
+    with pytest.raises(EngineError):
+        ops.add_rmsnorm(x, None, torch.ones(9, device=DEV), 1e-5, torch.float32)
+    with pytest.raises(EngineError):
+        ops.add_rmsnorm(x, None, torch.ones(8, device=DEV), 0.0, torch.float32)                  # src/operators.cpp:27
+    with pytest.raises(EngineError):
+        ops.gemm_generic(x.half(), torch.randn(5, 8, device=DEV).half(), None, torch.float16)    # float16 is not a storage type here
+    with pytest.raises(EngineError):
+        ops.attention_generic(torch.randn(2, 2 * 300, device=DEV), torch.zeros(1, 2, 1, 16, 300, device=DEV),
+                              torch.zeros(1, 1, dtype=torch.int32, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV),
+                              torch.zeros(2, dtype=torch.int32, device=DEV), 2, 1, 300, None, 1.0)   # head size above 256

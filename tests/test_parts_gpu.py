@@ -1,0 +1,273 @@
+"""Each part alone against its plain reference, and the generality of the parts: a mixer with state
+of its own, a position encoding that is no rotation, and an architecture of its own, all defined
+here and registered without a change to the engine's files; a layer order that names a layer twice
+and lets a run read another run's cache; a windowed attention whose pages come back."""
+import json
+import math
+import os
+from dataclasses import dataclass
+
+import pytest
+import torch
+
+from plain_llama import plain_attention, plain_linear, plain_rms_norm, plain_rope, plain_silu_mul
+from gpu_helpers import assert_close, load_plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+
+
+def part_weights(part_class, spec, prefix, dtype, seed):
+    from tlie_amd.weights import random_tensors
+    tensors = random_tensors(part_class.tensor_specs(spec, prefix), seed, std=0.2, norm_std=0.2, dtype=dtype)
+    return tensors, {name: tensor.to(DEV) for name, tensor in tensors.items()}
+
+
+class MixerHarness:
+    """A cache manager and step contexts around one mixer, nothing else of a model."""
+
+    def __init__(self, mixer, dtype, num_pages=40, page_size=8):
+        from tlie_amd.cache import CacheManager, RunNeed
+        self.mixer = mixer
+        self.cache = CacheManager([RunNeed(0, mixer.cache_need(), mixer.state_need())], page_size, num_pages, 4, dtype, DEV)
+
+    def run(self, items):
+        """items: [(request, x [n, hidden])]; returns the mixer's output rows per request."""
+        from tlie_amd.engine.step import StepEntry, build_context
+        from tlie_amd.ops import as_product
+        entries = []
+        for request, x in items:
+            if not self.cache.is_live(request):
+                self.cache.admit(request)
+            self.cache.reserve(request, x.shape[0])
+            entries.append(StepEntry(request, [0] * x.shape[0], []))
+        ctx = build_context(self.cache, entries, DEV)
+        out = as_product(self.mixer.forward(torch.cat([x for _, x in items]).contiguous(), ctx, self.cache.bindings[0])).dense()
+        for request, x in items:
+            self.cache.commit(request, x.shape[0])
+        self.cache.check()
+        return torch.split(out, [x.shape[0] for _, x in items])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_rms_norm_part(dtype):
+    from tlie_amd.config import PartSpec
+    from tlie_amd.parts.norm import RMSNorm
+    spec = PartSpec("rms_norm", {"size": 200, "eps": 3e-4})
+    host, device = part_weights(RMSNorm, spec, "n.", DT[dtype], 1)
+    part = RMSNorm(spec, DT[dtype], DEV)
+    part.load(device, "n.")
+    x = torch.randn(5, 200)
+    assert_close(part.forward(x.to(DEV)), plain_rms_norm(x, host["n.weight"].double(), 3e-4), TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_gated_mlp_part(dtype):
+    from tlie_amd.config import PartSpec
+    from tlie_amd.ops import as_product
+    from tlie_amd.parts.mlp import GatedMLP
+    spec = PartSpec("gated_mlp", {"hidden_size": 72, "intermediate_size": 200, "activation": "silu"})
+    host, device = part_weights(GatedMLP, spec, "m.", DT[dtype], 2)
+    part = GatedMLP(spec, DT[dtype], DEV)
+    part.load(device, "m.")
+    x = torch.randn(11, 72).to(DT[dtype])
+    got = as_product(part.forward(x.to(DEV), None)).dense()
+    hidden = plain_silu_mul(plain_linear(x.double(), host["m.gate_proj.weight"]), plain_linear(x.double(), host["m.up_proj.weight"]))
+    if dtype == "bfloat16":
+        hidden = hidden.to(torch.bfloat16).double()          # the activation between the two products is stored in bfloat16
+    assert_close(got, plain_linear(hidden, host["m.down_proj.weight"]), TOL[dtype])
+
+
+def plain_attention_part(x, host, prefix, nq, nkv, d, theta, window, bias, rot_dim=None):
+    tokens = x.shape[0]
+    def lin(name):
+        return plain_linear(x.double(), host[f"{prefix}{name}_proj.weight"], host.get(f"{prefix}{name}_proj.bias") if bias else None)
+    positions = torch.arange(tokens)
+    q, k, v = lin("q").view(tokens, nq, d), lin("k").view(tokens, nkv, d), lin("v").view(tokens, nkv, d)
+    if theta is not None:
+        rot = rot_dim or d
+        q = torch.cat([plain_rope(q[..., :rot], positions, theta), q[..., rot:]], dim=-1)
+        k = torch.cat([plain_rope(k[..., :rot], positions, theta), k[..., rot:]], dim=-1)
+    attended = plain_attention(q, k, v, window=window).reshape(tokens, nq * d)
+    return plain_linear(attended, host[prefix + "o_proj.weight"], host.get(prefix + "o_proj.bias") if bias else None)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", [
+    dict(hidden=40, nq=5, nkv=5, d=16, bias=False, window=None, theta=10000.0),        # plain multi-head
+    dict(hidden=72, nq=6, nkv=2, d=48, bias=True, window=None, theta=500000.0),
+    dict(hidden=64, nq=4, nkv=1, d=32, bias=False, window=11, theta=10000.0),          # a window; pages come back
+    dict(hidden=64, nq=2, nkv=2, d=64, bias=True, window=None, theta=None),            # no position encoding
+    dict(hidden=48, nq=3, nkv=1, d=32, bias=False, window=None, theta=10000.0, rot_dim=16),   # part of the head turns
+])
+def test_attention_part_whole_and_in_portions(dtype, case):
+    from tlie_amd.config import PartSpec
+    from tlie_amd.parts.attention import Attention
+    position = PartSpec("none") if case["theta"] is None else PartSpec("rotary", {
+        "head_dim": case["d"], "theta": case["theta"], **({"rot_dim": case["rot_dim"]} if "rot_dim" in case else {})})
+    spec = PartSpec("attention", {"hidden_size": case["hidden"], "num_heads": case["nq"], "num_kv_heads": case["nkv"],
+                                  "head_dim": case["d"], "bias": case["bias"], "window": case["window"], "position": position})
+    host, device = part_weights(Attention, spec, "a.", DT[dtype], 3)
+    part = Attention(spec, DT[dtype], DEV)
+    part.load(device, "a.")
+    tokens = 61
+    x = torch.randn(tokens, case["hidden"]).to(DT[dtype])
+    want = plain_attention_part(x, host, "a.", case["nq"], case["nkv"], case["d"], case["theta"], case["window"], case["bias"],
+                                case.get("rot_dim"))
+    harness = MixerHarness(part, DT[dtype])
+    (whole,) = harness.run([("w", x.to(DEV))])
+    assert_close(whole, want, TOL[dtype], "whole")
+    pieces, cursor = [], 0
+    for size in (9, 2, 1, 17, 1, 1, 8, 22):
+        other = torch.randn(3, case["hidden"]).to(DT[dtype]).to(DEV)            # another request beside it in the batch
+        out = harness.run([("other", other), ("p", x[cursor:cursor + size].to(DEV))])
+        pieces.append(out[1])
+        cursor += size
+    assert cursor == tokens
+    assert_close(torch.cat(pieces), want, TOL[dtype], "in portions")
+    if case["window"] is not None:
+        held = [page for page in harness.cache.page_list("p", 0) if page >= 0]
+        assert len(held) <= (case["window"] + 7) // 8 + 1, "pages a window has passed were not given back"
+
+
+# ---------------------------------------------------------------------------------------------------
+# Parts and an architecture defined by the test.
+
+def register_toys():
+    from tlie_amd import ops
+    from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run, TensorSpec
+    from tlie_amd.parts import Mixer, PositionEncoding, StateNeed
+    from tlie_amd.parts.linear import Linear
+    from tlie_amd.registry import register
+
+    @register("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """out[t] = W . mean(x[0..t]): the only thing carried from step to step is the running sum,
+        a state of fixed size per request."""
+
+        @classmethod
+        def tensor_specs(cls, spec, prefix):
+            return [TensorSpec(prefix + "mix.weight", (spec["hidden_size"], spec["hidden_size"]))]
+
+        def load(self, weights, prefix):
+            self.mix = Linear(weights[prefix + "mix.weight"], None, self.dtype)
+
+        def state_need(self):
+            return StateNeed((self.spec["hidden_size"],), torch.float32)
+
+        def forward(self, x, ctx, binding):
+            means = torch.empty_like(x, dtype=torch.float32)
+            starts = ctx.host["seq_start"]
+            for index in range(ctx.num_seqs):
+                begin, end, slot = int(starts[index]), int(starts[index + 1]), int(ctx.host["seq_slot"][index])
+                sums = torch.cumsum(x[begin:end].float(), dim=0) + binding.state[slot]
+                binding.state[slot] = sums[-1]
+                means[begin:end] = sums / (ctx.positions[begin:end].float() + 1.0)[:, None]
+            return self.mix(means.to(self.dtype).contiguous())
+
+    @register("position_encoding", "toy_scale_by_position")
+    class ScaleByPosition(PositionEncoding):
+        """Not a rotation: keys are scaled by 1 / (1 + position / 64)."""
+
+        def apply_qk(self, q, k, positions):
+            scale = (1.0 / (1.0 + positions.float() / 64.0))[:, None, None]
+            return q, (k.float() * scale).to(k.dtype)
+
+    @register("architecture", "ToyForCausalLM")
+    @dataclass(frozen=True)
+    class ToyConfig:
+        hidden_size: int
+        vocab_size: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["hidden_size"], raw["vocab_size"], raw["eps"])
+
+        def to_dict(self):
+            return {"architectures": ["ToyForCausalLM"], "hidden_size": self.hidden_size, "vocab_size": self.vocab_size, "eps": self.eps}
+
+        def to_spec(self):
+            norm = PartSpec("rms_norm", {"size": self.hidden_size, "eps": self.eps})
+            attention = PartSpec("attention", {"hidden_size": self.hidden_size, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                               "bias": False, "window": None, "position": PartSpec("toy_scale_by_position")})
+            mean = PartSpec("toy_running_mean", {"hidden_size": self.hidden_size})
+            mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 40, "activation": "silu"})
+            layers = (LayerSpec("model.layers.0.", "pre_norm", attention, mlp, norm, norm),
+                      LayerSpec("model.layers.1.", "pre_norm", mean, mlp, norm, norm))
+            # layer 0 runs three times: with a cache of its own, again with another cache of its own,
+            # and once more reading the first run's cache; the toy mixer's layer runs in between
+            runs = (Run(0, 0), Run(1, 1), Run(0, 2), Run(0, 0))
+            return ModelSpec("ToyForCausalLM", self.hidden_size, self.vocab_size, 128,
+                             PartSpec("token_embedding", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size}),
+                             layers, runs, norm,
+                             PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "tied": False}))
+    return ToyConfig
+
+
+def plain_toy_forward(raw, w, tokens):
+    """The toy architecture, whole sequence, from the plain functions."""
+    hidden, eps = raw["hidden_size"], raw["eps"]
+    count = len(tokens)
+    positions = torch.arange(count)
+    x = w["model.embed_tokens.weight"][tokens]
+    kept = {}
+
+    def attention_run(x, own_cache, read=None):
+        p = "model.layers.0."
+        normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)
+        q = plain_linear(normed, w[p + "self_attn.q_proj.weight"]).view(count, 2, 16)
+        k = plain_linear(normed, w[p + "self_attn.k_proj.weight"]).view(count, 1, 16) / (1.0 + positions.double() / 64.0)[:, None, None]
+        v = plain_linear(normed, w[p + "self_attn.v_proj.weight"]).view(count, 1, 16)
+        if own_cache is not None:
+            kept[own_cache] = (k, v)
+        else:
+            k, v = kept[read]
+        x = x + plain_linear(plain_attention(q, k, v).reshape(count, 32), w[p + "self_attn.o_proj.weight"])
+        return x + mlp(x, p)
+
+    def mlp(x, p):
+        normed = plain_rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
+        return plain_linear(plain_silu_mul(plain_linear(normed, w[p + "mlp.gate_proj.weight"]),
+                                           plain_linear(normed, w[p + "mlp.up_proj.weight"])), w[p + "mlp.down_proj.weight"])
+
+    x = attention_run(x, own_cache=0)
+    p = "model.layers.1."
+    normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)
+    means = torch.cumsum(normed, dim=0) / (positions.double() + 1.0)[:, None]
+    x = x + plain_linear(means, w[p + "self_attn.mix.weight"])
+    x = x + mlp(x, p)
+    x = attention_run(x, own_cache=2)
+    x = attention_run(x, own_cache=None, read=0)
+    return plain_linear(plain_rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+def test_toy_parts_register_build_and_step(tmp_path):
+    from tlie_amd import Engine, write_random_model
+    from gpu_helpers import Replayer
+    toy = register_toys()
+    config = toy(hidden_size=32, vocab_size=90, eps=1e-5)
+    write_random_model(str(tmp_path), config, seed=5, std=0.15, norm_std=0.1, dtype=torch.float32)
+    raw, weights = load_plain(str(tmp_path))
+    engine = Engine(str(tmp_path), dtype="float32", max_tokens=256, page_size=8, max_requests=3)
+    assert [binding.group for binding in engine.cache.bindings] == [0, None, 0, 0]
+    assert engine.cache.bindings[3].cache is engine.cache.bindings[0].cache and not engine.cache.bindings[3].writes
+    assert engine.cache.bindings[2].cache is not engine.cache.bindings[0].cache
+    assert engine.cache.bindings[1].state.shape == (3, 32)
+    tokens = [(7 * i * i + 3) % 90 for i in range(50)]
+    other = [(5 * i + 1) % 90 for i in range(23)]
+    want, want_other = plain_toy_forward(raw, weights, tokens), plain_toy_forward(raw, weights, other)
+    replay = Replayer(engine)
+    replay.step([("whole", tokens, list(range(50)))], end=["whole"])
+    assert_close(replay.logits_of("whole", range(50)), want, 2e-5, "whole")
+    # in portions, with another request beside it that ends and whose slot (and state row) is used again
+    replay.step([("a", tokens[:13], list(range(13))), ("b", other, list(range(23)))], end=["b"])
+    replay.step([("a", tokens[13:15], [0, 1]), ("c", other[:9], list(range(9)))])
+    replay.step([("c", other[9:], list(range(14))), ("a", tokens[15:16], [0])], end=["c"])
+    replay.step([("a", tokens[16:], list(range(34)))], end=["a"])
+    assert_close(replay.logits_of("a", range(50)), want, 2e-5, "in portions")
+    assert_close(replay.logits_of("b", range(23)), want_other, 2e-5, "beside it")
+    assert_close(replay.logits_of("c", range(23)), want_other, 2e-5, "in a slot that was used before")
+    assert engine.cache.free_slots == 3

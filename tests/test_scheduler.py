@@ -1,0 +1,175 @@
+"""The scheduler's decisions, on the CPU, with the real cache manager and a stand-in for the model
+(the next token is a function of the tokens so far, so recomputation after a preemption must give
+the same output as an undisturbed run)."""
+import pytest
+import torch
+
+from tlie_amd import EngineError, ErrorCode
+from tlie_amd.cache import CacheManager, RunNeed
+from tlie_amd.engine import Request, SamplingParams, Scheduler
+from tlie_amd.parts import KVCacheNeed
+
+
+def make(num_pages=16, page_size=4, max_requests=4, **kwargs):
+    cache = CacheManager([RunNeed(0, KVCacheNeed(1, 8))], page_size, num_pages, max_requests, torch.float32, "cpu",
+                         max_positions=kwargs.pop("max_positions", 64))
+    return cache, Scheduler(cache, max_positions=cache.max_positions, **kwargs)
+
+
+def fake_token(tokens):
+    return (sum(tokens) * 31 + len(tokens) * 7) % 97
+
+
+def drive(cache, scheduler, log=None, max_steps=500):
+    """Runs plans against the cache manager as the engine loop does."""
+    for _ in range(max_steps):
+        if not scheduler.has_work():
+            return
+        plan = scheduler.schedule()
+        assert plan, "no progress"
+        seen = set()
+        for item in plan:
+            assert item.request.id not in seen
+            seen.add(item.request.id)
+            assert item.first == cache.length(item.request.id) == item.request.computed
+        assert cache.can_reserve([(item.request.id, item.count) for item in plan])
+        for item in plan:
+            cache.reserve(item.request.id, item.count)
+            cache.commit(item.request.id, item.count)
+        if log is not None:
+            log.append([(item.request.id, item.first, item.count, item.samples) for item in plan])
+        sampled = [fake_token(item.request.tokens[:item.first + item.count]) for item in plan if item.samples]
+        scheduler.update(plan, sampled)
+        cache.check()
+    raise AssertionError("did not finish")
+
+
+def expected_output(prompt, count):
+    tokens, out = list(prompt), []
+    for _ in range(count):
+        out.append(fake_token(tokens))
+        tokens.append(out[-1])
+    return out
+
+
+def test_prompt_is_cut_under_the_budget_then_decodes():
+    cache, scheduler = make(max_tokens_per_step=8)
+    request = Request("a", list(range(1, 20)), SamplingParams(max_tokens=3))
+    scheduler.add(request)
+    log = []
+    drive(cache, scheduler, log)
+    assert log == [[("a", 0, 8, False)], [("a", 8, 8, False)], [("a", 16, 3, True)], [("a", 19, 1, True)], [("a", 20, 1, True)]]
+    assert request.generated == expected_output(request.prompt, 3) and request.finish_reason == "length"
+    assert cache.free_pages() == [16] and cache.free_slots == 4       # everything came back
+    # the last sampled token is never fed back (app/reference_cli.cpp:103): 19 + 2 positions were cached
+    assert scheduler.stats["prefill_tokens"] == 19 and scheduler.stats["decode_tokens"] == 2
+
+
+def test_decodes_first_then_fills_with_prompt_portions_fifo():
+    cache, scheduler = make(max_tokens_per_step=6, num_pages=32)
+    a = Request("a", [1, 2, 3], SamplingParams(max_tokens=4))
+    b = Request("b", list(range(10, 21)), SamplingParams(max_tokens=2))
+    c = Request("c", [5, 6], SamplingParams(max_tokens=2))
+    for request in (a, b, c):
+        scheduler.add(request)
+    log = []
+    drive(cache, scheduler, log)
+    assert log[0] == [("a", 0, 3, True), ("b", 0, 3, False)]            # first come first served under 6 tokens
+    assert log[1] == [("a", 3, 1, True), ("b", 3, 5, False)]            # the decoding request comes first
+    assert log[2] == [("a", 4, 1, True), ("b", 8, 3, True), ("c", 0, 2, True)]
+    for request in (a, b, c):
+        assert request.generated == expected_output(request.prompt, request.params.max_tokens)
+
+
+def test_admission_waits_for_a_slot():
+    cache, scheduler = make(max_requests=2, num_pages=32)
+    requests = [Request(i, [i + 1, i + 2], SamplingParams(max_tokens=3)) for i in range(4)]
+    for request in requests:
+        scheduler.add(request)
+    log = []
+    drive(cache, scheduler, log)
+    assert [entry[0] for entry in log[0]] == [0, 1]
+    first_of = {rid: index for index, step in enumerate(log) for (rid, first, _, _) in step if first == 0}
+    assert first_of[2] == 3 and first_of[3] == 3                          # after the first two finished (3 outputs)
+    for request in requests:
+        assert request.generated == expected_output(request.prompt, 3)
+
+
+def test_requests_that_can_never_fit_are_refused():
+    cache, scheduler = make(num_pages=4, page_size=4, max_positions=64)
+    with pytest.raises(EngineError) as caught:
+        scheduler.add(Request("big", list(range(1, 17)), SamplingParams(max_tokens=2)))     # needs 17 positions, pool holds 16
+    assert caught.value.code == ErrorCode.OUT_OF_MEMORY
+    scheduler.add(Request("fits", list(range(1, 16)), SamplingParams(max_tokens=2)))         # 16 positions
+    with pytest.raises(EngineError) as caught:
+        scheduler.add(Request("long", list(range(60)), SamplingParams(max_tokens=5)))
+    assert caught.value.code == ErrorCode.OUT_OF_BOUNDS                   # app/reference_cli.cpp:72-75
+    with pytest.raises(EngineError):
+        scheduler.add(Request("empty", [], SamplingParams(max_tokens=5)))
+    with pytest.raises(EngineError):
+        scheduler.add(Request("zero", [1], SamplingParams(max_tokens=0)))
+    with pytest.raises(EngineError):
+        scheduler.add(Request("p", [1], SamplingParams(top_p=0.0)))
+    drive(cache, scheduler)
+
+
+def test_pages_run_out_while_decoding_the_last_admitted_is_preempted():
+    # 6 pages of 4: two requests of 9-token prompts take 3 pages each (positions 0..11); when they
+    # grow past 12 positions each needs a fourth page and none is free.
+    cache, scheduler = make(num_pages=6, page_size=4)
+    a = Request("a", list(range(1, 10)), SamplingParams(max_tokens=8))
+    b = Request("b", list(range(21, 30)), SamplingParams(max_tokens=8))
+    scheduler.add(a)
+    scheduler.add(b)
+    log = []
+    drive(cache, scheduler, log)
+    assert scheduler.stats["preemptions"] >= 1 and b.preemptions >= 1 and a.preemptions == 0   # the victim is the last admitted
+    assert a.generated == expected_output(a.prompt, 8) and b.generated == expected_output(b.prompt, 8)
+    # "b" was recomputed from position 0, its prompt and what it had generated so far: in all it ran
+    # more tokens than an undisturbed run of 9 + 7
+    restarts = [index for index, step in enumerate(log) if index > 0 for (rid, first, _, _) in step if rid == "b" and first == 0]
+    assert restarts
+    assert sum(count for step in log for (rid, _, count, _) in step if rid == "b") > 16
+    assert sum(count for step in log for (rid, _, count, _) in step if rid == "a") == 16
+    assert cache.free_pages() == [6] and cache.free_slots == 4
+
+
+def test_prompts_that_block_each_other_are_untangled():
+    # two prompts of 28 tokens (7 pages each) in a pool of 10: cut into portions of 8 they take
+    # pages turn by turn until neither can go on; the later one is preempted, the earlier finishes.
+    cache, scheduler = make(num_pages=10, page_size=4, max_tokens_per_step=16, chunk_size=8)
+    a = Request("a", list(range(1, 29)), SamplingParams(max_tokens=2))
+    b = Request("b", list(range(31, 59)), SamplingParams(max_tokens=2))
+    scheduler.add(a)
+    scheduler.add(b)
+    drive(cache, scheduler)
+    assert a.generated == expected_output(a.prompt, 2) and b.generated == expected_output(b.prompt, 2)
+    assert b.preemptions >= 1 and a.preemptions == 0
+
+
+def test_more_decoders_than_the_budget_rotate():
+    cache, scheduler = make(num_pages=32, max_requests=4, max_seqs_per_step=2, max_tokens_per_step=64)
+    requests = [Request(i, [i + 1], SamplingParams(max_tokens=5)) for i in range(4)]
+    for request in requests:
+        scheduler.add(request)
+    log = []
+    drive(cache, scheduler, log)
+    assert all(len(step) <= 2 for step in log)
+    for request in requests:
+        assert request.generated == expected_output(request.prompt, 5)       # nobody starves
+
+
+def test_abort_and_eos():
+    cache, scheduler = make()
+    a = Request("a", [1, 2, 3], SamplingParams(max_tokens=50))
+    scheduler.add(a)
+    scheduler.update(plan := scheduler.schedule(), [fake_token(a.prompt)])
+    for item in plan:
+        pass
+    assert scheduler.abort("a") and a.finish_reason == "aborted" and not scheduler.has_work()
+    assert not scheduler.abort("a")
+    cache2, scheduler2 = make(eos_token_id=fake_token([4, 5]))
+    b = Request("b", [4, 5], SamplingParams(max_tokens=50, stop_on_eos=True))
+    scheduler2.add(b)
+    drive(cache2, scheduler2)
+    assert b.finish_reason == "eos" and len(b.generated) == 1

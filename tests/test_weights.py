@@ -1,0 +1,140 @@
+"""The weight store.  Cases follow the reference's unit tests of its store
+(tests/unit_tests.cpp:114-171: valid file, missing tensor, shape mismatch, wrong byte count,
+truncated file), on safetensors files instead of its own format."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from tlie_amd import EngineError, ErrorCode, LlamaConfig, write_random_model
+from tlie_amd.models import expected_tensors
+from tlie_amd.weights import SafetensorsFile, WeightStore, random_tensors, to_kept_precision, write_safetensors
+
+TINY = dict(model_type="llama", hidden_size=32, intermediate_size=48, num_hidden_layers=2, num_attention_heads=4,
+            num_key_value_heads=2, max_position_embeddings=64, vocab_size=40, rms_norm_eps=1e-5)
+
+
+def code_of(call):
+    with pytest.raises(EngineError) as caught:
+        call()
+    return caught.value
+
+
+def test_round_trip_against_the_library(tmp_path):
+    tensors = {"a": torch.randn(3, 5), "b.c": torch.randn(7).bfloat16(), "ids": torch.arange(6, dtype=torch.int64).view(2, 3),
+               "empty": torch.zeros(0, 4)}
+    mine = str(tmp_path / "mine.safetensors")
+    write_safetensors(mine, tensors, {"k": "v"})
+    theirs = load_file(mine)
+    for name, tensor in tensors.items():
+        assert torch.equal(theirs[name], tensor)
+    lib = str(tmp_path / "lib.safetensors")
+    save_file(tensors, lib)
+    file = SafetensorsFile(lib)
+    for name, tensor in tensors.items():
+        assert torch.equal(file.tensor(name), tensor) and file.tensor(name).dtype == tensor.dtype
+
+
+def test_random_model_loads_and_is_seeded(tmp_path):
+    config = LlamaConfig.from_dict(TINY)
+    one, two, other = (str(tmp_path / name) for name in ("one", "two", "other"))
+    write_random_model(one, config, seed=3)
+    write_random_model(two, config, seed=3)
+    write_random_model(other, config, seed=4)
+    specs = expected_tensors(config.to_spec())
+    a = WeightStore(one).load(specs, torch.bfloat16, "cpu")
+    b = WeightStore(two).load(specs, torch.bfloat16, "cpu")
+    c = WeightStore(other).load(specs, torch.bfloat16, "cpu")
+    assert set(a) == {spec.name for spec in specs}
+    assert all(torch.equal(a[name], b[name]) for name in a)
+    assert not torch.equal(a["lm_head.weight"], c["lm_head.weight"])
+    assert json.load(open(os.path.join(one, "config.json")))["hidden_size"] == 32
+    # a tensor's values depend on (seed, name) only, not on which other tensors are drawn
+    alone = random_tensors([s for s in specs if s.name == "model.norm.weight"], seed=3)
+    assert torch.equal(alone["model.norm.weight"], a["model.norm.weight"])
+    assert abs(a["model.norm.weight"].float().mean().item() - 1.0) < 0.05           # norms are drawn around 1
+    assert abs(a["lm_head.weight"].float().std().item() - 0.02) < 0.005
+
+
+def test_kept_precision():
+    assert to_kept_precision(torch.ones(2, dtype=torch.float16), torch.bfloat16).dtype == torch.bfloat16
+    assert to_kept_precision(torch.ones(2, dtype=torch.bfloat16), torch.bfloat16).dtype == torch.bfloat16
+    assert to_kept_precision(torch.ones(2, dtype=torch.float32), torch.bfloat16).dtype == torch.float32   # 32-bit stays
+    assert to_kept_precision(torch.ones(2, dtype=torch.int64), torch.bfloat16).dtype == torch.int32        # integer tables
+    assert to_kept_precision(torch.ones(2, dtype=torch.bfloat16), torch.float32).dtype == torch.float32
+    assert code_of(lambda: to_kept_precision(torch.ones(2), torch.float16)).code == ErrorCode.INVALID_DTYPE
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    config = LlamaConfig.from_dict(TINY)
+    specs = expected_tensors(config.to_spec())
+    tensors = random_tensors(specs, seed=0)
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(32, 31).bfloat16()
+    tensors["model.layers.0.extra.weight"] = torch.zeros(2).bfloat16()
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(4)         # a stored buffer: ignored
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    error = code_of(lambda: WeightStore(str(tmp_path)).load(specs, torch.bfloat16, "cpu"))
+    assert error.code == ErrorCode.INVALID_SHAPE
+    for piece in ("2 missing", "model.layers.1.mlp.up_proj.weight", "model.norm.weight", "1 unexpected",
+                  "model.layers.0.extra.weight", "1 with a wrong shape", "stored [32, 31], expected [32, 32]"):
+        assert piece in error.message, piece
+    assert "inv_freq" not in error.message
+
+
+def test_tied_model_may_carry_its_head(tmp_path):
+    config = LlamaConfig.from_dict(dict(TINY, tie_word_embeddings=True))
+    specs = expected_tensors(config.to_spec())
+    tensors = random_tensors(specs, seed=0)
+    assert "lm_head.weight" not in tensors
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    WeightStore(str(tmp_path)).validate(specs)
+    tensors["lm_head.weight"] = torch.zeros(40, 32).bfloat16()
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    WeightStore(str(tmp_path)).validate(specs)
+
+
+def test_broken_files(tmp_path):
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.IO
+    path = str(tmp_path / "model.safetensors")
+    write_safetensors(path, {"w": torch.randn(4, 4)})
+    raw = open(path, "rb").read()
+    open(path, "wb").write(raw[:-5])                                   # truncated (tests/unit_tests.cpp:166-170)
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
+    open(path, "wb").write(raw + b"\0\0\0\0")                          # trailing bytes
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
+    open(path, "wb").write(raw[:4])
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
+
+    def with_header(header, payload=b"\0" * 64):
+        text = json.dumps(header).encode()
+        open(path, "wb").write(struct.pack("<Q", len(text)) + text + payload)
+    with_header({"w": {"dtype": "F32", "shape": [4, 4], "data_offsets": [0, 60]}})          # bytes do not fit the shape
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_SHAPE
+    with_header({"w": {"dtype": "F8_E4M3", "shape": [64], "data_offsets": [0, 64]}})
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_DTYPE
+    with_header({"w": {"dtype": "F32", "shape": [8], "data_offsets": [0, 32]}, "v": {"dtype": "F32", "shape": [8], "data_offsets": [16, 48]}})
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT     # overlap
+    text = b'{"w": {"dtype": "F32", "shape": [8], "data_offsets": [0, 32]}, "w": {"dtype": "F32", "shape": [8], "data_offsets": [32, 64]}}'
+    open(path, "wb").write(struct.pack("<Q", len(text)) + text + b"\0" * 64)
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT     # duplicate name
+    open(path, "wb").write(struct.pack("<Q", 1 << 40) + b"{}")
+    assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
+
+
+def test_sharded_folder(tmp_path):
+    config = LlamaConfig.from_dict(TINY)
+    specs = expected_tensors(config.to_spec())
+    tensors = random_tensors(specs, seed=1)
+    names = sorted(tensors)
+    half = len(names) // 2
+    write_safetensors(str(tmp_path / "model-00001-of-00002.safetensors"), {n: tensors[n] for n in names[:half]})
+    write_safetensors(str(tmp_path / "model-00002-of-00002.safetensors"), {n: tensors[n] for n in names[half:]})
+    weight_map = {n: ("model-00001-of-00002.safetensors" if i < half else "model-00002-of-00002.safetensors") for i, n in enumerate(names)}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
+    loaded = WeightStore(str(tmp_path)).load(specs, torch.float32, "cpu")
+    assert all(torch.equal(loaded[n], tensors[n].float()) for n in names)

@@ -19,6 +19,8 @@ from ..errors import EngineError, ErrorCode, invalid_argument
 from ..models.builder import build_model, expected_tensors
 from ..registry import config_from_dict
 from ..weights.store import WeightStore
+from ..sampling.sampler import Sampler
+from .scheduler import Request, SamplingParams, Scheduler
 from .step import ModelRunner, StepEntry
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
@@ -65,3 +67,38 @@ class Engine:
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         return self.runner.step(entries)
+
+    # ---- generation -------------------------------------------------------------------------------
+    def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,
+                 top_p: float = 1.0, seed: int = 0, stop_on_eos: bool = False, max_tokens_per_step: int = 2048,
+                 max_seqs_per_step: int | None = None, chunk_size: int | None = None) -> list[list[int]]:
+        """Token ids in, generated token ids out, one list per prompt.  Request i samples with
+        seed + i.  All prompts run together under the scheduler (continuous batching, prompts cut
+        into portions under the token budget)."""
+        scheduler = Scheduler(self.cache, max_tokens_per_step=max_tokens_per_step,
+                              max_seqs_per_step=max_seqs_per_step or self.cache.max_requests, chunk_size=chunk_size,
+                              max_positions=self.spec.max_positions, eos_token_id=self.spec.eos_token_id)
+        requests = []
+        for index, prompt in enumerate(prompts):
+            params = SamplingParams(max_tokens=max_tokens, temperature=temperature, top_p=top_p, seed=seed + index,
+                                    stop_on_eos=stop_on_eos)
+            request = Request(id=("generate", index), prompt=[int(token) for token in prompt], params=params)
+            scheduler.add(request)
+            requests.append(request)
+        self.run(scheduler)
+        return [request.generated for request in requests]
+
+    def run(self, scheduler: Scheduler) -> None:
+        """The engine loop: plan a step, run it, sample, record; until nothing is left."""
+        sampler = Sampler(self.device)
+        while scheduler.has_work():
+            plan = scheduler.schedule()
+            if not plan:
+                raise EngineError(ErrorCode.OUT_OF_MEMORY, "no request can make progress with the pages that are free")
+            entries = [StepEntry(item.request.id, item.request.tokens[item.first:item.first + item.count],
+                                 [item.count - 1] if item.samples else []) for item in plan]
+            logits = self.step(entries)
+            sampling = [item for item in plan if item.samples]
+            tokens = sampler.sample(logits, [item.request.params for item in sampling],
+                                    [len(item.request.generated) for item in sampling])
+            scheduler.update(plan, tokens)

@@ -17,7 +17,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import ABSENT, CacheManager
-from ..errors import invalid_argument, out_of_bounds
+from ..errors import invalid_argument, out_of_bounds, out_of_memory
 
 
 @dataclass
@@ -87,54 +87,7 @@ class ModelRunner:
                 raise out_of_bounds(f"request {entry.request!r} would pass the model's {limit} positions")
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        cache = self.cache
-        counts = [len(entry.tokens) for entry in entries]
-        total, seqs = sum(counts), len(entries)
-        first = [cache.length(entry.request) for entry in entries]
-        tokens = np.concatenate([np.asarray(entry.tokens, dtype=np.int32) for entry in entries])
-        positions = np.concatenate([np.arange(start, start + n, dtype=np.int32) for start, n in zip(first, counts)])
-        token_seq = np.repeat(np.arange(seqs, dtype=np.int32), counts)
-        seq_start = np.zeros(seqs + 1, dtype=np.int32)
-        seq_start[1:] = np.cumsum(counts)
-        want_rows = np.asarray([seq_start[index] + int(place) for index, entry in enumerate(entries) for place in entry.want],
-                               dtype=np.int32)
-        host = {
-            "tokens": tokens, "positions": positions, "token_seq": token_seq,
-            "no_slots": np.full(total, -1, dtype=np.int32), "seq_start": seq_start,
-            "seq_first_pos": np.asarray(first, dtype=np.int32),
-            "seq_len": np.asarray([start + n for start, n in zip(first, counts)], dtype=np.int32),
-            "seq_slot": np.asarray([cache.slot(entry.request) for entry in entries], dtype=np.int32),
-            "want_rows": want_rows,
-        }
-        group_shapes = []
-        for group in range(len(cache.groups)):
-            lists = [cache.page_list(entry.request, group) for entry in entries]
-            width = max(1, max(len(pages) for pages in lists))
-            table = np.zeros((seqs, width), dtype=np.int32)
-            for row, pages in enumerate(lists):
-                table[row, :len(pages)] = [page if page != ABSENT else 0 for page in pages]
-            slot_map = np.concatenate([np.asarray(cache.rows(entry.request, group, start, n), dtype=np.int32)
-                                       for entry, start, n in zip(entries, first, counts)])
-            host[f"block_table{group}"] = table
-            host[f"slot_map{group}"] = slot_map
-            group_shapes.append(width)
-        # one transfer for all of it
-        names = list(host)
-        flat = np.concatenate([host[name].ravel() for name in names])
-        device_flat = torch.from_numpy(flat).to(self.device, non_blocking=False)
-        views, cursor = {}, 0
-        for name in names:
-            size = host[name].size
-            views[name] = device_flat[cursor:cursor + size].view(host[name].shape)
-            cursor += size
-        groups = [GroupView(views[f"block_table{group}"], views[f"slot_map{group}"], width)
-                  for group, width in enumerate(group_shapes)]
-        return StepContext(
-            num_tokens=total, num_seqs=seqs, num_wanted=int(want_rows.size), max_new=max(counts),
-            max_context=int(host["seq_len"].max()), tokens=views["tokens"], positions=views["positions"],
-            token_seq=views["token_seq"], no_slots=views["no_slots"], seq_start=views["seq_start"],
-            seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
-            want_rows=views["want_rows"], groups=groups, host=host)
+        return build_context(self.cache, entries, self.device)
 
     # ---- the step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -144,7 +97,6 @@ class ModelRunner:
         self._validate(entries)
         wanted = [(entry.request, len(entry.tokens)) for entry in entries]
         if not self.cache.can_reserve(wanted):
-            from ..errors import out_of_memory
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         for request, count in wanted:
             self.cache.reserve(request, count)
@@ -153,3 +105,56 @@ class ModelRunner:
         for request, count in wanted:
             self.cache.commit(request, count)
         return logits
+
+
+def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> StepContext:
+    """The step's arrays for entries whose pages are reserved: built on the host, sent in one
+    transfer."""
+    counts = [len(entry.tokens) for entry in entries]
+    total, seqs = sum(counts), len(entries)
+    first = [cache.length(entry.request) for entry in entries]
+    tokens = np.concatenate([np.asarray(entry.tokens, dtype=np.int32) for entry in entries])
+    positions = np.concatenate([np.arange(start, start + n, dtype=np.int32) for start, n in zip(first, counts)])
+    token_seq = np.repeat(np.arange(seqs, dtype=np.int32), counts)
+    seq_start = np.zeros(seqs + 1, dtype=np.int32)
+    seq_start[1:] = np.cumsum(counts)
+    want_rows = np.asarray([seq_start[index] + int(place) for index, entry in enumerate(entries) for place in entry.want],
+                           dtype=np.int32)
+    host = {
+        "tokens": tokens, "positions": positions, "token_seq": token_seq,
+        "no_slots": np.full(total, -1, dtype=np.int32), "seq_start": seq_start,
+        "seq_first_pos": np.asarray(first, dtype=np.int32),
+        "seq_len": np.asarray([start + n for start, n in zip(first, counts)], dtype=np.int32),
+        "seq_slot": np.asarray([cache.slot(entry.request) for entry in entries], dtype=np.int32),
+        "want_rows": want_rows,
+    }
+    group_shapes = []
+    for group in range(len(cache.groups)):
+        lists = [cache.page_list(entry.request, group) for entry in entries]
+        width = max(1, max(len(pages) for pages in lists))
+        table = np.zeros((seqs, width), dtype=np.int32)
+        for row, pages in enumerate(lists):
+            table[row, :len(pages)] = [page if page != ABSENT else 0 for page in pages]
+        slot_map = np.concatenate([np.asarray(cache.rows(entry.request, group, start, n), dtype=np.int32)
+                                   for entry, start, n in zip(entries, first, counts)])
+        host[f"block_table{group}"] = table
+        host[f"slot_map{group}"] = slot_map
+        group_shapes.append(width)
+    # one transfer for all of it
+    names = list(host)
+    flat = np.concatenate([host[name].ravel() for name in names])
+    device_flat = torch.from_numpy(flat).to(device, non_blocking=False)
+    views, cursor = {}, 0
+    for name in names:
+        size = host[name].size
+        views[name] = device_flat[cursor:cursor + size].view(host[name].shape)
+        cursor += size
+    groups = [GroupView(views[f"block_table{group}"], views[f"slot_map{group}"], width)
+              for group, width in enumerate(group_shapes)]
+    return StepContext(
+        num_tokens=total, num_seqs=seqs, num_wanted=int(want_rows.size), max_new=max(counts),
+        max_context=int(host["seq_len"].max()), tokens=views["tokens"], positions=views["positions"],
+        token_seq=views["token_seq"], no_slots=views["no_slots"], seq_start=views["seq_start"],
+        seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
+        want_rows=views["want_rows"], groups=groups, host=host)
+
