@@ -1,0 +1,172 @@
+"""Measures decoding and prefill of the TinyLlama 1.1B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--dtype bfloat16]
+
+A step is one decode step of the whole batch.  The batch's requests are first prefilled so that
+after the warm-up and the K timed steps their length is `context`; then W untimed and exactly K
+timed steps run, each through the engine's own step function and sampler (greedy), and one JSON
+line is printed.  `value` is decoded tokens per second.  The same line carries the prefill of a
+2,048-token prompt, the decode step's share of the HBM roofline, and decoding at batch 1 and 64.
+
+Peaks are the MI355X's published ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bfloat16, 157.3
+TFLOP/s for float32.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+HBM_PEAK = 8.0e12
+MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+# configs[2] of BASELINE.json: TinyLlama 1.1B
+TINYLLAMA = dict(model_type="llama", architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=5632,
+                 num_hidden_layers=22, num_attention_heads=32, num_key_value_heads=4, max_position_embeddings=2048,
+                 vocab_size=32000, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False, attention_bias=False,
+                 hidden_act="silu", bos_token_id=1, eos_token_id=2, torch_dtype="bfloat16")
+
+
+def weight_bytes_per_step(cfg, itemsize):
+    """Bytes of weights a decode step reads: every matrix once, the norms, the head; of the
+    embedding table only the batch's rows (not counted)."""
+    h, i, d = cfg["hidden_size"], cfg["intermediate_size"], cfg["hidden_size"] // cfg["num_attention_heads"]
+    qd, kvd = cfg["num_attention_heads"] * d, cfg["num_key_value_heads"] * d
+    per_layer = (qd + 2 * kvd) * h + h * qd + 2 * i * h + h * i + 2 * h
+    return (cfg["num_hidden_layers"] * per_layer + h + cfg["vocab_size"] * h) * itemsize
+
+
+def kv_bytes_per_token(cfg, itemsize):
+    d = cfg["hidden_size"] // cfg["num_attention_heads"]
+    return 2 * cfg["num_key_value_heads"] * d * cfg["num_hidden_layers"] * itemsize
+
+
+def prefill_flops(cfg, tokens):
+    h, i, d = cfg["hidden_size"], cfg["intermediate_size"], cfg["hidden_size"] // cfg["num_attention_heads"]
+    nq = cfg["num_attention_heads"]
+    qd, kvd = nq * d, cfg["num_key_value_heads"] * d
+    linear = 2 * tokens * cfg["num_hidden_layers"] * ((qd + 2 * kvd) * h + h * qd + 3 * i * h)
+    attention = cfg["num_hidden_layers"] * 4 * nq * d * tokens * (tokens + 1) // 2
+    head = 2 * cfg["vocab_size"] * h
+    return linear + attention + head
+
+
+def time_decode(engine, torch, batch, context, steps, warmup, vocab):
+    """Prefills `batch` requests, runs warmup + steps decode steps ending at `context` positions;
+    returns seconds for the timed steps."""
+    from tlie_amd import StepEntry
+    from tlie_amd.engine import SamplingParams
+    from tlie_amd.sampling import Sampler
+    sampler = Sampler(engine.device)
+    params = [SamplingParams() for _ in range(batch)]
+    prompt_len = context - steps - warmup
+    generator = torch.Generator().manual_seed(batch)
+    requests = [("bench", index) for index in range(batch)]
+    tokens = []
+    for request in requests:
+        prompt = torch.randint(0, vocab, (prompt_len,), generator=generator).tolist()
+        engine.admit(request)
+        logits = engine.step([StepEntry(request, prompt, [prompt_len - 1])])
+        tokens.append(sampler.sample(logits, params[:1], [0])[0])
+
+    def run(count):
+        nonlocal tokens
+        for index in range(count):
+            logits = engine.step([StepEntry(request, [token], [0]) for request, token in zip(requests, tokens)])
+            tokens = sampler.sample(logits, params, [index] * batch)
+    run(warmup)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    run(steps)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    for request in requests:
+        engine.finish(request)
+    return elapsed
+
+
+def time_prefill(engine, torch, tokens, vocab, repeats=3):
+    from tlie_amd import StepEntry
+    generator = torch.Generator().manual_seed(tokens)
+    prompt = torch.randint(0, vocab, (tokens,), generator=generator).tolist()
+    best = None
+    for _ in range(repeats + 1):
+        engine.admit("prefill")
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        logits = engine.step([StepEntry("prefill", prompt, [tokens - 1])])
+        logits.argmax(-1).item()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        engine.finish("prefill")
+        best = elapsed if best is None else min(best, elapsed)       # the first run also warms up
+    return best
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=128)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--context", type=int, default=2048)
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the configuration has (named in the record)")
+    parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
+        return 2
+    import torch
+    from tlie_amd import Engine
+    cfg = dict(TINYLLAMA)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    if args.context > cfg["max_position_embeddings"] or args.steps + args.warmup >= args.context:
+        print("context must fit the model's positions and exceed steps + warmup")
+        return 2
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    vocab = cfg["vocab_size"]
+    most = max(args.batch, 1 if args.no_points else 64)
+    engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=most * args.context + 2048,
+                    page_size=16, max_requests=most + 1)
+
+    elapsed = time_decode(engine, torch, args.batch, args.context, args.steps, args.warmup, vocab)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = args.batch * args.steps / elapsed
+    mean_context = args.context - args.steps / 2
+    step_bytes = weight_bytes_per_step(cfg, itemsize) + args.batch * mean_context * kv_bytes_per_token(cfg, itemsize)
+    achieved = step_bytes / (elapsed / args.steps)
+    record = {
+        "metric": "decode tok/s at batch 8, context 2048 (TinyLlama 1.1B shape)", "value": value, "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {"model": "TinyLlama-1.1B shape", "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
+                   "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                   "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "ffn": cfg["intermediate_size"],
+                   "vocab": vocab, "global_batch": args.batch, "seq_len": args.context, "page_size": 16,
+                   "parallelism": "single GPU"},
+        "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK},
+    }
+    if not args.no_points:
+        prefill_tokens = 2048
+        seconds = time_prefill(engine, torch, prefill_tokens, vocab)
+        record["prefill"] = {"value": prefill_tokens / seconds, "tokens": prefill_tokens, "ms": seconds * 1e3,
+                             "frac": prefill_flops(cfg, prefill_tokens) / seconds / MFMA_PEAK[args.dtype]}
+        points = {}
+        for batch in (1, 64):
+            steps = min(args.steps, 64)
+            seconds = time_decode(engine, torch, batch, args.context, steps, 4, vocab)
+            points[f"decode_b{batch}"] = batch * steps / seconds
+        record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

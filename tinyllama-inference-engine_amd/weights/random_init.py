@@ -18,27 +18,29 @@ from ..config.spec import TensorSpec
 from .safetensors_io import write_safetensors
 
 
-def _generator(seed: int, name: str) -> torch.Generator:
+def _generator(seed: int, name: str, device="cpu") -> torch.Generator:
     digest = hashlib.sha256(f"{seed}:{name}".encode("utf-8")).digest()
-    generator = torch.Generator(device="cpu")
+    generator = torch.Generator(device=device)
     generator.manual_seed(int.from_bytes(digest[:8], "little") & 0x7FFF_FFFF_FFFF_FFFF)
     return generator
 
 
 def random_tensors(specs: list[TensorSpec], seed: int, std: float = 0.02, norm_std: float = 0.01,
-                   dtype: torch.dtype = torch.bfloat16) -> dict[str, torch.Tensor]:
+                   dtype: torch.dtype = torch.bfloat16, device="cpu") -> dict[str, torch.Tensor]:
+    """Drawn on `device`; the values of a (seed, name) are the same on every run on one kind of
+    device, but differ between the CPU's and the GPU's generators."""
     out = {}
     for spec in specs:
         if spec.optional:
             continue
-        generator = _generator(seed, spec.name)
-        values = torch.randn(spec.shape, generator=generator, dtype=torch.float32)
+        generator = _generator(seed, spec.name, device)
+        values = torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device)
         if spec.init == "normal":
             values = values * std
         elif spec.init == "norm":
             values = 1.0 + values * norm_std
         elif spec.init == "zeros":
-            values = torch.zeros(spec.shape)
+            values = torch.zeros(spec.shape, device=device)
         else:
             raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
         out[spec.name] = values.to(dtype)
