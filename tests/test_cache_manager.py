@@ -92,7 +92,7 @@ def test_groups_by_need_and_shared_caches():
     assert [group.window for group in cache.groups] == [None, 6]
     assert [b.group for b in cache.bindings] == [0, 1, 0, None, 1]
     assert cache.bindings[2].cache is cache.bindings[0].cache and not cache.bindings[2].writes and cache.bindings[0].writes
-    assert cache.bindings[1].cache.shape == (6, 2, 1, 4, 16) and cache.bindings[4].cache.shape == (6, 2, 2, 4, 8)
+    assert cache.bindings[1].cache.shape == (6, 2, 1, 4 * 16) and cache.bindings[4].cache.shape == (6, 2, 2, 4 * 8)
     with pytest.raises(EngineError):
         CacheManager([RunNeed(0, KVCacheNeed(2, 8)), RunNeed(0, KVCacheNeed(1, 8))], 4, 6, 2, torch.float32, "cpu")
     # the windowed group gives pages back as the request grows; the full group keeps them

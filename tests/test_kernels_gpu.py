@@ -116,17 +116,21 @@ def test_gemm_is_true_32_bit():
 
 def build_cache(k, v, page_size, dtype, shuffle_seed=0, extra_pages=3):
     """Puts one sequence's keys and values [T, nkv, d] on pages in shuffled physical order.
-    Returns (cache [pages, 2, nkv, page_size, d], block table row)."""
+    Returns (cache [pages, 2, nkv, page_size * d], block table row).  Per page and kv head the keys
+    lie as [row][dim], the values transposed as [dim][row].  Rows that hold no token of the sequence
+    hold NaN: a kernel that lets them reach a result shows it."""
     tokens, nkv, d = k.shape
     blocks = (tokens + page_size - 1) // page_size
     order = list(range(blocks + extra_pages))
     random.Random(shuffle_seed).shuffle(order)
-    cache = torch.full((blocks + extra_pages, 2, nkv, page_size, d), 7.5).to(dtype)     # stale rows hold a loud value
+    keys = torch.full((blocks + extra_pages, nkv, page_size, d), float("nan"))
+    values = torch.full((blocks + extra_pages, nkv, d, page_size), float("nan"))
     for position in range(tokens):
         page, row = order[position // page_size], position % page_size
-        cache[page, 0, :, row] = k[position].to(dtype)
-        cache[page, 1, :, row] = v[position].to(dtype)
-    return cache, order[:blocks]
+        keys[page, :, row, :] = k[position]
+        values[page, :, :, row] = v[position]
+    cache = torch.stack([keys.reshape(-1, nkv, page_size * d), values.reshape(-1, nkv, page_size * d)], dim=1).to(dtype)
+    return cache.contiguous(), order[:blocks]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -206,15 +210,15 @@ def test_rope_cache(dtype):
     # the reference's golden vector (data/golden/operators.json:25-63): 2 q heads, 1 kv head, d = 4, position 7
     qkv = torch.tensor([[0.1, 0.2, 0.3, 0.4, -0.5, 0.6, -0.7, 0.8, 0.9, -1.0, 1.1, -1.2, 5.0, 6.0, 7.0, 8.0]], device=DEV)
     inv_freq = torch.pow(torch.tensor(10000.0), -2.0 * torch.arange(2, dtype=torch.float32) / 4.0).to(DEV)
-    cache = torch.zeros(3, 2, 1, 4, 4, device=DEV)
+    cache = torch.zeros(3, 2, 1, 4 * 4, device=DEV)
     q = ops.rope_cache(ops.Product(qkv, 1), torch.tensor([7], dtype=torch.int32, device=DEV),
                        torch.tensor([2 * 4 + 1], dtype=torch.int32, device=DEV), inv_freq, 4, cache, 2, 1, 4, torch.float32)
     want_q = torch.tensor([-0.12170576304197311, 0.17153306305408478, 0.2918693423271179, 0.41300898790359497,
                            0.08293947577476501, 0.5425763726234436, -0.8562248945236206, 0.8400065302848816])
     want_k = torch.tensor([-0.044173240661621094, -0.9136196374893188, 1.4205803871154785, -1.267004132270813])
     assert torch.allclose(q.cpu().flatten(), want_q, atol=1e-6, rtol=0)
-    assert torch.allclose(cache[2, 0, 0, 1].cpu(), want_k, atol=1e-6, rtol=0)
-    assert torch.equal(cache[2, 1, 0, 1].cpu(), torch.tensor([5.0, 6.0, 7.0, 8.0]))      # the value is stored unrotated
+    assert torch.allclose(cache[2, 0, 0].view(4, 4)[1].cpu(), want_k, atol=1e-6, rtol=0)   # keys: [row][dim]
+    assert torch.equal(cache[2, 1, 0].view(4, 4)[:, 1].cpu(), torch.tensor([5.0, 6.0, 7.0, 8.0]))   # values: [dim][row], unrotated
     assert float(cache.abs().sum()) == pytest.approx(float(want_k.abs().sum()) + 26.0, rel=1e-5)   # nothing else was written
 
     # other sizes, split partial sums, far positions (the reference tests position 4095: tests/cuda/kernel_tests.cu:144-146)
@@ -225,7 +229,7 @@ def test_rope_cache(dtype):
     slots = torch.tensor([3, 12, -1, 40, 41, 7, 0, 63, 20], dtype=torch.int32)
     theta = 500000.0
     inv_freq = torch.pow(torch.tensor(theta), -2.0 * torch.arange(d // 2, dtype=torch.float32) / d).to(DEV)
-    cache = torch.full((8, 2, nkv, page, d), -3.0).to(DT[dtype]).to(DEV)
+    cache = torch.full((8, 2, nkv, page * d), -3.0).to(DT[dtype]).to(DEV)
     q = ops.rope_cache(ops.Product(parts.to(DEV), 2), positions.to(DEV), slots.to(DEV), inv_freq, d, cache, nq, nkv, d, DT[dtype])
     total = parts.double().sum(0)
     want_q = plain_rope(total[:, :nq * d].view(tokens, nq, d), positions, theta)
@@ -233,21 +237,23 @@ def test_rope_cache(dtype):
     want_v = total[:, (nq + nkv) * d:].view(tokens, nkv, d)
     assert rel_err(q.view(tokens, nq, d), want_q) < TOL[dtype]
     cache = cache.cpu()
+    keys, values = cache[:, 0].view(8, nkv, page, d), cache[:, 1].view(8, nkv, d, page)
     written = torch.zeros(8, page, dtype=torch.bool)
     for t in range(tokens):
         if slots[t] < 0:
             continue
         page_index, row = int(slots[t]) // page, int(slots[t]) % page
         written[page_index, row] = True
-        assert rel_err(cache[page_index, 0, :, row], want_k[t]) < TOL[dtype]
-        assert rel_err(cache[page_index, 1, :, row], want_v[t]) < TOL[dtype]
+        assert rel_err(keys[page_index, :, row, :], want_k[t]) < TOL[dtype]
+        assert rel_err(values[page_index, :, :, row], want_v[t]) < TOL[dtype]
     for page_index in range(8):
         for row in range(page):
             if not written[page_index, row]:
-                assert float((cache[page_index, :, :, row].float() + 3.0).abs().max()) == 0.0
+                assert float((keys[page_index, :, row, :].float() + 3.0).abs().max()) == 0.0
+                assert float((values[page_index, :, :, row].float() + 3.0).abs().max()) == 0.0
     # no rotation table: q and k pass through
     plain_q = ops.rope_cache(ops.Product(parts[0].to(DEV).contiguous(), 1), positions.to(DEV), slots.to(DEV), None, 0,
-                             torch.zeros(8, 2, nkv, page, d, dtype=DT[dtype], device=DEV), nq, nkv, d, DT[dtype])
+                             torch.zeros(8, 2, nkv, page * d, dtype=DT[dtype], device=DEV), nq, nkv, d, DT[dtype])
     assert rel_err(plain_q, parts[0][:, :nq * d]) < TOL[dtype]
 
 
@@ -265,6 +271,146 @@ def test_kernels_refuse_what_they_do_not_take():
     with pytest.raises(EngineError):
         ops.gemm_generic(x.half(), torch.randn(5, 8, device=DEV).half(), None, torch.float16)    # float16 is not a storage type here
     with pytest.raises(EngineError):
-        ops.attention_generic(torch.randn(2, 2 * 300, device=DEV), torch.zeros(1, 2, 1, 16, 300, device=DEV),
+        ops.attention_generic(torch.randn(2, 2 * 300, device=DEV), torch.zeros(1, 2, 1, 16 * 300, device=DEV),
                               torch.zeros(1, 1, dtype=torch.int32, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV),
                               torch.zeros(2, dtype=torch.int32, device=DEV), 2, 1, 300, None, 1.0)   # head size above 256
+
+
+# ---- the bfloat16 kernels on the matrix cores ---------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(1, 40, 64), (3, 177, 176), (16, 2560, 2048), (17, 100, 520), (33, 64, 5632),
+                                   (64, 515, 1000), (8, 32000, 2048), (5, 16, 8)])
+def test_gemm_skinny(shape):
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(n)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    b = torch.randn(n).bfloat16()
+    want = plain_linear(x.double(), w.double(), b.double())
+    product = ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV))
+    assert product.data.shape == (product.nsplit, m, n) and product.data.dtype == torch.float32
+    assert rel_err(product.dense(), want) < 5e-6                          # bfloat16 products are exact in float32; only the sums round
+    for split_len in (64, 128, 512, 8192):
+        product = ops.gemm_skinny(x.to(DEV), w.to(DEV), None, split_len=split_len)
+        assert product.nsplit == (k + split_len - 1) // split_len
+        assert rel_err(product.dense(), plain_linear(x.double(), w.double())) < 5e-6
+    # a row's result does not depend on how many other rows come with it
+    if m > 1:
+        alone = ops.gemm_skinny(x[:1].to(DEV).contiguous(), w.to(DEV), b.to(DEV), split_len=128).data
+        together = ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV), split_len=128).data
+        assert torch.equal(alone[:, 0], together[:, 0])                      # every partial sum, bit for bit
+
+
+def test_gemm_skinny_refuses():
+    from tlie_amd import EngineError, ops
+    w = torch.randn(32, 64, device=DEV).bfloat16()
+    with pytest.raises(EngineError):
+        ops.gemm_skinny(torch.randn(65, 64, device=DEV).bfloat16(), w, None)                  # too many rows
+    with pytest.raises(EngineError):
+        ops.gemm_skinny(torch.randn(2, 12, device=DEV).bfloat16(), torch.randn(8, 12, device=DEV).bfloat16(), None)   # K % 8
+    with pytest.raises(EngineError):
+        ops.gemm_skinny(torch.randn(2, 64, device=DEV), w, None)                              # float32
+    assert not ops.gemm_skinny_takes(torch.randn(2, 12, device=DEV).bfloat16(), torch.randn(8, 12, device=DEV).bfloat16())
+
+
+def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0):
+    """One sequence through the tiled kernel: q rows for the positions in token_list (default all)."""
+    from tlie_amd import ops
+    import numpy as np
+    tokens, nq, d = q.shape
+    nkv = k.shape[1]
+    cache, pages = build_cache(k, v, page, torch.bfloat16, shuffle_seed=shuffle_seed)
+    token_list = list(range(tokens)) if token_list is None else token_list
+    # the step brings a run of consecutive positions of the one sequence
+    assert token_list == list(range(token_list[0], token_list[0] + len(token_list)))
+    table = torch.tensor([[0] * len(pages), pages], dtype=torch.int32, device=DEV)
+    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv)
+    tiles[:, 0] = 1                                                            # the sequence is row 1 of the table
+    out = ops.attention_mfma(q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV), cache.to(DEV), table,
+                             torch.from_numpy(tiles).to(DEV), torch.tensor(token_list, dtype=torch.int32, device=DEV),
+                             nq, nkv, d, window, 1.0 / math.sqrt(d), nsplit)
+    return out.view(len(token_list), nq, d)
+
+
+@pytest.mark.parametrize("case", [
+    dict(tokens=3, nq=2, nkv=1, d=16, page=16),
+    dict(tokens=77, nq=6, nkv=3, d=48, page=16),
+    dict(tokens=300, nq=5, nkv=5, d=80, page=32),
+    dict(tokens=700, nq=8, nkv=1, d=128, page=16),
+    dict(tokens=333, nq=4, nkv=2, d=16, page=8, window=37),
+    dict(tokens=130, nq=3, nkv=1, d=256, page=64),
+    dict(tokens=200, nq=32, nkv=4, d=64, page=16),
+    dict(tokens=150, nq=40, nkv=2, d=32, page=4, window=50),          # 20 heads a group: more than one tile per token
+    dict(tokens=97, nq=7, nkv=7, d=112, page=16),
+])
+def test_attention_mfma(case):
+    tokens, nq, nkv, d, page = case["tokens"], case["nq"], case["nkv"], case["d"], case["page"]
+    window = case.get("window")
+    torch.manual_seed(tokens)
+    q, k, v = torch.randn(tokens, nq, d), torch.randn(tokens, nkv, d), torch.randn(tokens, nkv, d)
+    want = plain_attention(rounded(q, torch.bfloat16), rounded(k, torch.bfloat16), rounded(v, torch.bfloat16), window=window)
+    whole = run_attention_mfma(q, k, v, page, window, 1, shuffle_seed=tokens)
+    assert rel_err(whole, want) < TOL["bfloat16"]
+    # the last token alone (a decode step), its key range cut in parts that are merged
+    for nsplit in (1, 2, 5):
+        last = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=tokens)
+        assert rel_err(last[0], want[-1]) < TOL["bfloat16"], f"nsplit {nsplit}"
+    # a portion in the middle that starts and ends off the page and block boundaries
+    first, count = max(0, tokens // 2 - 9), min(21, tokens - max(0, tokens // 2 - 9))
+    portion = run_attention_mfma(q, k, v, page, window, 1, token_list=list(range(first, first + count)), shuffle_seed=tokens)
+    assert rel_err(portion, want[first:first + count]) < TOL["bfloat16"]
+    split_portion = run_attention_mfma(q, k, v, page, window, 3, token_list=list(range(first, first + count)), shuffle_seed=tokens)
+    assert rel_err(split_portion, want[first:first + count]) < TOL["bfloat16"]
+
+
+def test_attention_mfma_finds_one_key_among_hundreds():
+    tokens, nq, nkv, d, page = 600, 4, 2, 32, 16
+    torch.manual_seed(1)
+    base_k, v = torch.randn(tokens, nkv, d) * 0.1, torch.randn(tokens, nkv, d)
+    q = torch.randn(tokens, nq, d) * 0.1
+    direction = torch.zeros(d)
+    direction[3] = 1.0
+    q[tokens - 1] += 12.0 * direction
+    for window, needle, inside in [(None, 0, True), (None, 15, True), (None, 16, True), (None, 31, True), (None, 32, True),
+                                   (None, 511, True), (None, 598, True), (None, 599, True), (100, 500, True), (100, 499, False),
+                                   (16, 584, True), (16, 583, False)]:
+        k = base_k.clone()
+        k[needle] += 12.0 * direction
+        for nsplit in (1, 4):
+            got = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=needle)[0].float().cpu()
+            wanted_rows = v[needle].bfloat16().float().repeat_interleave(nq // nkv, dim=0)
+            hit = (got - wanted_rows).abs().max().item() < 0.05
+            assert hit == inside, f"window {window}, needle at {needle}, nsplit {nsplit}: {'missed' if inside else 'seen'}"
+
+
+def test_attention_mfma_mixed_step():
+    """Three sequences in one step: a portion of a prompt, one decoded token, a whole short prompt;
+    each must equal what it gives alone."""
+    from tlie_amd import ops
+    import numpy as np
+    nq, nkv, d, page = 6, 2, 64, 16
+    torch.manual_seed(9)
+    lengths, brings = [90, 200, 11], [(50, 40), (199, 1), (0, 11)]             # (first position, count) brought by the step
+    qs, ks, vs = zip(*[(torch.randn(n, nq, d), torch.randn(n, nkv, d), torch.randn(n, nkv, d)) for n in lengths])
+    caches, tables, offset = [], [], 0
+    for index in range(3):
+        cache, pages = build_cache(ks[index], vs[index], page, torch.bfloat16, shuffle_seed=index)
+        tables.append([page_index + offset for page_index in pages])
+        offset += cache.shape[0]
+        caches.append(cache)
+    width = max(len(t) for t in tables)
+    table = torch.tensor([t + [0] * (width - len(t)) for t in tables], dtype=torch.int32, device=DEV)
+    q_rows = torch.cat([qs[i][first:first + count] for i, (first, count) in enumerate(brings)]).bfloat16().reshape(-1, nq * d)
+    positions = torch.tensor([p for first, count in brings for p in range(first, first + count)], dtype=torch.int32, device=DEV)
+    seq_start = np.cumsum([0] + [count for _, count in brings])
+    tiles = torch.from_numpy(ops.attention_tiles(seq_start, nq // nkv)).to(DEV)
+    for nsplit in (1, 3):
+        out = ops.attention_mfma(q_rows.contiguous().to(DEV), torch.cat(caches).to(DEV), table, tiles, positions, nq, nkv, d,
+                                 None, 1.0 / math.sqrt(d), nsplit).view(-1, nq, d)
+        cursor = 0
+        for index, (first, count) in enumerate(brings):
+            want = plain_attention(rounded(qs[index], torch.bfloat16), rounded(ks[index], torch.bfloat16),
+                                   rounded(vs[index], torch.bfloat16))[first:first + count]
+            assert rel_err(out[cursor:cursor + count], want) < TOL["bfloat16"], f"sequence {index}, nsplit {nsplit}"
+            cursor += count

@@ -11,7 +11,8 @@ Groups.  Runs of layers whose caches have the same need (every key kept, or a wi
 positions) form a group.  A group has its own allocator and, per request, its own list of pages:
 entry b of the list is the page that holds positions b * page_size ... (b + 1) * page_size - 1.
 The page number is shared by all runs of the group: each run has its own pool tensor
-[pages, 2, kv heads, page_size, head_dim], indexed by the same page number.  A windowed group
+[pages, 2, kv heads, page_size * head_dim] (per page and kv head the keys lie as [row][dim], the values
+transposed, as [dim][row]), indexed by the same page number.  A windowed group
 gives a page back as soon as every position on it is out of every later token's window.
 
 Nothing is cleared when pages or slots come back: a kernel reads only rows that were written for
@@ -84,7 +85,8 @@ class CacheManager:
                 index = group_of_window[need.kv.window]
                 self.groups[index].owners.append(run)
                 group_of_run[run] = index
-                pools[run] = torch.empty((num_pages, 2, need.kv.num_kv_heads, page_size, need.kv.head_dim),
+                # zeros once, at creation: rows that were never written then hold finite values
+                pools[run] = torch.zeros((num_pages, 2, need.kv.num_kv_heads, page_size * need.kv.head_dim),
                                          dtype=dtype, device=device)
         for run, need in enumerate(needs):
             binding = Binding()

@@ -14,7 +14,8 @@
 
 namespace tlie {
 
-// q: [tokens][nq][d]; cache: [pages][2][nkv][page_size][d]; out: [tokens][nq][d].
+// q: [tokens][nq][d]; cache: [pages][2][nkv][page_size * d], keys [row][dim], values [dim][row];
+// out: [tokens][nq][d].
 // token_seq[t]: row of the block table; positions[t]: absolute position of the token.
 // window <= 0: all keys 0..pos; otherwise keys pos-window+1..pos.
 template <typename T>
@@ -65,8 +66,8 @@ __global__ void attention_generic_kernel(const T* __restrict__ q, const T* __res
       for (int jj = max(0, lo - start); jj < last; ++jj) {
         const int key_pos = start + jj;
         const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset + head_offset +
-                         static_cast<size_t>(key_pos % page_size) * d;
-        acc += prob[jj] * to_float(value[threadIdx.x]);
+                         static_cast<size_t>(threadIdx.x) * page_size + key_pos % page_size;
+        acc += prob[jj] * to_float(*value);
       }
     }
     __syncthreads();

@@ -1,0 +1,138 @@
+// y = x . W^T for few rows of x (a decode batch, or a short step): bfloat16 in, float partial
+// sums out, on the matrix cores.  The kernel is bound by reading W once from HBM, so W goes
+// straight from global memory into the MFMA operand registers (every element of W is used by one
+// wave only); x, which every wave needs, is staged through LDS.
+//
+// reference: every product of the reference's device path is one library call per projection
+// (GemmFp16RowMajor, src/cuda/kernels.cu:342-368), also for one token.  A matrix of 2048 rows
+// gives a 256-CU part too few waves when each wave takes whole rows, so K is split over
+// `nsplit` workgroups in y and the partial sums [nsplit, M, N] are left to the consumer (the
+// norm, rotation or activation kernel that reads them next) to add up.
+//
+// v_mfma_f32_16x16x32_bf16: operand A = 16 rows of W x 32 k, operand B = 16 rows of x x 32 k,
+// C[w row][x row].  Lane l supplies row (l & 15) and the 8 k values of group (l >> 4).  Which k
+// values a slot stands for is free as long as A and B agree, so a lane takes 16 consecutive k of
+// its row per 64-wide step (two MFMAs): its loads are 32 contiguous bytes and a row's four lanes
+// read 128 contiguous bytes.
+#include "common.h"
+
+namespace tlie {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+union Pack16 {
+  uint4 u;
+  bf16x8 v;
+};
+
+constexpr int kSkinnyThreads = 256;          // 4 waves, 16 rows of W each
+constexpr int kSkinnyRowsPerBlock = 64;
+constexpr int kSkinnyPad = 8;                // bf16 elements of padding per LDS row (16 bytes): rows fall on different banks
+
+// NT: tiles of 16 rows of x (M <= 16 * NT).  CHUNK: k values staged in LDS at a time.
+// split_len: k values per split (multiple of 64).  K % 8 == 0.
+template <int NT, int CHUNK>
+__global__ void __launch_bounds__(kSkinnyThreads)
+gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
+                   float* __restrict__ y, int M, int N, int K, int split_len) {
+  constexpr int kStride = CHUNK + kSkinnyPad;
+  constexpr int kSteps = CHUNK / 64;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[NT * 16 * kStride];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int split = blockIdx.y;
+  const int k_begin = split * split_len, k_end = min(K, k_begin + split_len);
+  const int strip_row = blockIdx.x * kSkinnyRowsPerBlock + wave * 16;
+  const int group = lane >> 4;
+  const bool active = strip_row < N;
+  const int row = min(strip_row + (lane & 15), N - 1);
+  const uint16_t* w_row = w + static_cast<size_t>(row) * K;
+
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (int c0 = k_begin; c0 < k_end; c0 += CHUNK) {
+    const int c1 = min(k_end, c0 + CHUNK);
+    // this wave's part of W for the chunk: issued first, in flight while x is staged
+    Pack16 a[kSteps][2];
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      const int k = c0 + s * 64 + group * 16;
+      a[s][0].u = (active && k < c1) ? *reinterpret_cast<const uint4*>(w_row + k) : make_uint4(0, 0, 0, 0);
+      a[s][1].u = (active && k + 8 < c1) ? *reinterpret_cast<const uint4*>(w_row + k + 8) : make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();                         // the previous chunk's reads of xs are done
+    constexpr int kVectors = CHUNK / 8;
+    for (int i = threadIdx.x; i < NT * 16 * kVectors; i += kSkinnyThreads) {
+      const int token = i / kVectors, k = c0 + (i % kVectors) * 8;
+      uint4 value = make_uint4(0, 0, 0, 0);
+      if (token < M && k < c1) value = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * K + k);
+      *reinterpret_cast<uint4*>(xs + token * kStride + (k - c0)) = value;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      if (c0 + s * 64 >= c1) break;          // the same for every lane
+      const int offset = s * 64 + group * 16;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const uint16_t* x_row = xs + (t * 16 + (lane & 15)) * kStride + offset;
+        Pack16 b0, b1;
+        b0.u = *reinterpret_cast<const uint4*>(x_row);
+        b1.u = *reinterpret_cast<const uint4*>(x_row + 8);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][0].v, b0.v, acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][1].v, b1.v, acc[t], 0, 0, 0);
+      }
+    }
+  }
+  if (!active) return;
+  // acc[t][j] = y[token t*16 + (lane & 15)][strip_row + group*4 + j]
+  const int n0 = strip_row + group * 4;
+  float add[4] = {0.f, 0.f, 0.f, 0.f};
+  if (bias != nullptr && split == 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (n0 + j < N) add[j] = bf16_bits_to_float(bias[n0 + j]);
+  }
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int token = t * 16 + (lane & 15);
+    if (token >= M) continue;
+    float* out = y + (static_cast<size_t>(split) * M + token) * N + n0;
+    if ((N & 3) == 0 && n0 + 3 < N) {
+      *reinterpret_cast<float4*>(out) = make_float4(acc[t][0] + add[0], acc[t][1] + add[1], acc[t][2] + add[2], acc[t][3] + add[3]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (n0 + j < N) out[j] = acc[t][j] + add[j];
+    }
+  }
+}
+
+}  // namespace tlie
+
+using namespace tlie;
+
+// x [M, K], w [N, K], bias [N] or null: bfloat16.  y: float [nsplit, M, N] with
+// nsplit = ceil(K / split_len).  M <= 64, K % 8 == 0, split_len % 64 == 0.
+extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, float* y, int M, int N, int K,
+                                int split_len, void* stream) {
+  if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) != 0 || split_len <= 0 || (split_len & 63) != 0) return kBadArgument;
+  const int nsplit = (K + split_len - 1) / split_len;
+  const int tiles = (M + 15) / 16;
+  const int nt = tiles <= 1 ? 1 : (tiles == 2 ? 2 : 4);
+  const dim3 grid((N + kSkinnyRowsPerBlock - 1) / kSkinnyRowsPerBlock, nsplit);
+  if (grid.y > 65535) return kBadArgument;
+  hipStream_t s = (hipStream_t)stream;
+  const uint16_t* xp = (const uint16_t*)x;
+  const uint16_t* wp = (const uint16_t*)w;
+  const uint16_t* bp = (const uint16_t*)bias;
+  if (nt == 1)
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
+  else if (nt == 2)
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
+  else
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 256>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
+  return launch_status();
+}

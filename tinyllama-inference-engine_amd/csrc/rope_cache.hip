@@ -11,7 +11,8 @@
 namespace tlie {
 
 // qkv: [nsplit][tokens][(nq + 2 nkv) * d], columns ordered q heads | k heads | v heads.
-// q_out: [tokens][nq * d].  cache: [pages][2][nkv][page_size][d], K at index 0, V at 1.
+// q_out: [tokens][nq * d].  cache: [pages][2][nkv][page_size * d]: keys at index 0 as [row][dim],
+// values at index 1 transposed, [dim][row] (the attention kernels read 4 consecutive rows of one dim).
 // slot_map[t] = page * page_size + row of token t, or -1: nothing is written for that token.
 // rot_dim <= d, even: dimensions from rot_dim on are copied unrotated.  inv_freq may be null
 // (no rotation at all).
@@ -60,11 +61,12 @@ __global__ void rope_cache_kernel(const D* __restrict__ qkv, int nsplit, size_t 
       cache_row[(head - nq) * head_stride + e] = from_float<A>(result);
     }
   }
-  if (cache_row) {
-    A* v_row = cache_row + static_cast<size_t>(nkv) * head_stride;
+  if (slot >= 0) {
+    A* v_page = cache + static_cast<size_t>(slot / page_size) * page_stride + static_cast<size_t>(nkv) * head_stride +
+                slot % page_size;
     for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
       const int head = item / d, e = item % d;
-      v_row[head * head_stride + e] = from_float<A>(value((nq + nkv + head) * d + e));
+      v_page[head * head_stride + static_cast<size_t>(e) * page_size] = from_float<A>(value((nq + nkv + head) * d + e));
     }
   }
 }

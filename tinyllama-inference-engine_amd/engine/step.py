@@ -54,6 +54,20 @@ class StepContext:
     want_rows: torch.Tensor        # int32 [num_wanted] token indices
     groups: list[GroupView]
     host: dict                     # the same arrays as numpy, by name
+    _tiles: dict = field(default_factory=dict)
+
+    def attention_tiles(self, groups_per_kv: int, num_kv_heads: int):
+        """The tiled attention kernel's work list for this step (made once per group size), and
+        into how many parts each tile's key range is cut: as many as it takes to give a step of few
+        tiles about a thousand waves, each part at least 128 keys long."""
+        if groups_per_kv not in self._tiles:
+            from ..ops import attention_tiles
+            tiles = attention_tiles(self.host["seq_start"], groups_per_kv)
+            self._tiles[groups_per_kv] = torch.from_numpy(tiles).to(self.tokens.device)
+        tiles = self._tiles[groups_per_kv]
+        waves = tiles.shape[0] * num_kv_heads
+        nsplit = max(1, min((1024 + waves - 1) // waves, self.max_context // 128))
+        return tiles, nsplit
 
 
 class ModelRunner:

@@ -156,13 +156,21 @@ def silu_mul(gate_up: Product, out_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def _check_cache(cache: torch.Tensor, num_kv_heads: int, head_dim: int, what: str) -> int:
+    """cache: [pages, 2, nkv, page_size * d]; per page and kv head the keys lie as [row][dim] and
+    the values transposed, [dim][row].  Returns the page size."""
+    if cache.dim() != 4 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[3] % head_dim != 0:
+        raise invalid_shape(f"{what}: cache {list(cache.shape)} is not [pages, 2, nkv, page_size * d]")
+    return cache.shape[3] // head_dim
+
+
 def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
                rot_dim: int, cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                act_dtype: torch.dtype) -> torch.Tensor:
     """Rotates q and k, returns q [T, nq * d], writes k and v into the cache rows of `slot_map`.
 
-    cache: [pages, 2, nkv, page_size, d].  slot_map[t] = page * page_size + row, or -1 to skip.
-    The slot map comes from the cache manager, which hands out only rows of pages it owns."""
+    slot_map[t] = page * page_size + row, or -1 to skip.  The slot map comes from the cache
+    manager, which hands out only rows of pages it owns."""
     _check_product(qkv, "qkv")
     _device_tensor(positions, "positions", torch.int32)
     _device_tensor(slot_map, "slot_map", torch.int32)
@@ -172,8 +180,7 @@ def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, in
         raise invalid_shape(f"rope_cache: qkv width {qkv.cols} is not (nq + 2 nkv) * d")
     if positions.shape != (tokens,) or slot_map.shape != (tokens,):
         raise invalid_shape("rope_cache: positions and slot_map need one entry per token")
-    if cache.dim() != 5 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[4] != head_dim:
-        raise invalid_shape(f"rope_cache: cache {list(cache.shape)} is not [pages, 2, nkv, page_size, d]")
+    page_size = _check_cache(cache, num_kv_heads, head_dim, "rope_cache")
     if inv_freq is not None:
         _device_tensor(inv_freq, "inv_freq", torch.float32)
         if rot_dim % 2 != 0 or not 0 < rot_dim <= head_dim or inv_freq.shape != (rot_dim // 2,):
@@ -184,7 +191,7 @@ def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, in
     _check(library().tlie_rope_cache(_ptr(qkv.data), dtype_code(qkv.data.dtype), qkv.nsplit,
                                      ctypes.c_longlong(qkv.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
                                      rot_dim, _ptr(q_out), _ptr(cache), dtype_code(act_dtype), tokens, num_heads,
-                                     num_kv_heads, head_dim, cache.shape[3], _stream()), "rope_cache")
+                                     num_kv_heads, head_dim, page_size, _stream()), "rope_cache")
     return q_out
 
 
@@ -201,8 +208,7 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     tokens = q.shape[0]
     if q.shape != (tokens, num_heads * head_dim):
         raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
-    if cache.dim() != 5 or cache.shape[1] != 2 or cache.shape[2] != num_kv_heads or cache.shape[4] != head_dim:
-        raise invalid_shape(f"attention: cache {list(cache.shape)} is not [pages, 2, nkv, page_size, d]")
+    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention")
     if block_table.dim() != 2 or token_seq.shape != (tokens,) or positions.shape != (tokens,):
         raise invalid_shape("attention: block_table must be [sequences, max_blocks], token_seq and positions [tokens]")
     if num_heads % num_kv_heads != 0:
@@ -210,7 +216,7 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     out = torch.empty_like(q)
     _check(library().tlie_attention_generic(_ptr(q), _ptr(cache), dtype_code(q.dtype), _ptr(block_table),
                                             block_table.shape[1], _ptr(token_seq), _ptr(positions), _ptr(out), tokens,
-                                            num_heads, num_kv_heads, head_dim, cache.shape[3],
+                                            num_heads, num_kv_heads, head_dim, page_size,
                                             int(window) if window else 0, ctypes.c_float(scale), _stream()),
            "attention_generic")
     return out
@@ -255,4 +261,101 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p:
         return out
     _check(library().tlie_sample(_ptr(logits), rows, logits.shape[1], _ptr(temperature), _ptr(top_p), _ptr(seed),
                                  _ptr(counter), _ptr(out), _stream()), "sample")
+    return out
+
+
+# ---- bfloat16 kernels on the matrix cores ---------------------------------------------------------
+SKINNY_MAX_ROWS = 64
+_SKINNY_WAVES = 2048          # waves a skinny product is cut into at least, when K allows
+
+
+def skinny_split_len(rows: int, out_features: int, in_features: int) -> int:
+    """How many k values one split takes: enough splits that the product fills the chip's 256 CUs
+    with several waves each, never fewer than 128 k values (two 64-wide steps) per split, and
+    fewer splits for more rows, whose partial sums cost traffic of their own."""
+    strips = (out_features + 15) // 16
+    target = _SKINNY_WAVES if rows <= 16 else (_SKINNY_WAVES // 2 if rows <= 32 else _SKINNY_WAVES // 4)
+    splits = max(1, min((target + strips - 1) // strips, in_features // 128))
+    length = (in_features + splits - 1) // splits
+    return max(64, (length + 63) // 64 * 64)
+
+
+def gemm_skinny_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
+            and weight.shape[1] % 8 == 0)
+
+
+def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, split_len: int | None = None) -> Product:
+    """y = x . W^T (+ bias) for at most 64 rows of bfloat16 x: float partial sums [nsplit, M, N]."""
+    _device_tensor(x, "x", torch.bfloat16)
+    _device_tensor(weight, "weight", torch.bfloat16)
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise invalid_shape(f"gemm_skinny: x {list(x.shape)} and weight {list(weight.shape)} do not fit")
+    rows, (out_features, in_features) = x.shape[0], weight.shape
+    if not 0 < rows <= SKINNY_MAX_ROWS or in_features % 8 != 0:
+        raise invalid_argument(f"gemm_skinny takes 1..{SKINNY_MAX_ROWS} rows and an inner size that is a multiple of 8")
+    if bias is not None:
+        _device_tensor(bias, "bias", torch.bfloat16)
+        if bias.shape != (out_features,):
+            raise invalid_shape("gemm_skinny: bias needs one entry per output")
+    split_len = split_len or skinny_split_len(rows, out_features, in_features)
+    if split_len <= 0 or split_len % 64 != 0:
+        raise invalid_argument("gemm_skinny: a split's length must be a positive multiple of 64")
+    nsplit = (in_features + split_len - 1) // split_len
+    out = torch.empty((nsplit, rows, out_features), dtype=torch.float32, device=x.device)
+    _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), rows, out_features, in_features,
+                                      split_len, _stream()), "gemm_skinny")
+    return Product(out, nsplit)
+
+
+def attention_tiles(seq_start, groups_per_kv: int):
+    """The work list of the tiled attention kernel for a step, on the host: for every sequence,
+    tiles of 16 columns, a column being a (token, query head of one group) pair.
+    seq_start: the step's cumulative token counts [S + 1].  Returns an int32 array [tiles, 4]:
+    (sequence, its first token's index in the step, its number of tokens, the tile's first column)."""
+    import numpy as np
+    rows = []
+    for seq in range(len(seq_start) - 1):
+        first, count = int(seq_start[seq]), int(seq_start[seq + 1] - seq_start[seq])
+        for col0 in range(0, count * groups_per_kv, 16):
+            rows.append((seq, first, count, col0))
+    return np.asarray(rows, dtype=np.int32).reshape(-1, 4)
+
+
+def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
+    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= 256 and page_size % 4 == 0
+
+
+def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
+                   positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
+                   scale: float, nsplit: int = 1) -> torch.Tensor:
+    """Causal attention of every token of the step over its sequence's cache, bfloat16.
+
+    tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
+    positions: every tile's sequence is a row of block_table, its tokens are rows of q).  nsplit > 1
+    cuts every tile's key range into that many parts that run side by side and are merged."""
+    _device_tensor(q, "q", torch.bfloat16)
+    _device_tensor(cache, "cache", torch.bfloat16)
+    _device_tensor(block_table, "block_table", torch.int32)
+    _device_tensor(tiles, "tiles", torch.int32)
+    _device_tensor(positions, "positions", torch.int32)
+    tokens = q.shape[0]
+    if q.shape != (tokens, num_heads * head_dim):
+        raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
+    page_size = _check_cache(cache, num_kv_heads, head_dim, "attention")
+    if block_table.dim() != 2 or positions.shape != (tokens,) or tiles.dim() != 2 or tiles.shape[1] != 4 or tiles.shape[0] == 0:
+        raise invalid_shape("attention: block_table must be [sequences, max_blocks], positions [tokens], tiles [n, 4]")
+    if num_heads % num_kv_heads != 0:
+        raise invalid_shape("attention: the number of heads must be a multiple of the number of kv heads")
+    if not attention_mfma_takes(q.dtype, head_dim, page_size):
+        raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a multiple of 4 rows")
+    out = torch.empty_like(q)
+    part_o = part_ml = None
+    if nsplit > 1:
+        part_o = torch.empty((tokens * num_heads * nsplit, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((tokens * num_heads * nsplit, 2), dtype=torch.float32, device=q.device)
+    _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
+                                         tiles.shape[0], _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
+                                         tokens, num_heads, num_kv_heads, head_dim, page_size,
+                                         int(window) if window else 0, ctypes.c_float(scale), _stream()), "attention_mfma")
     return out

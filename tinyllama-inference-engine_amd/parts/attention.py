@@ -74,8 +74,14 @@ class Attention(Mixer):
         inv_freq, rot_dim = table if table is not None else (None, 0)
         q = ops.rope_cache(qkv, ctx.positions, slot_map, inv_freq, rot_dim, binding.cache, self.nq, self.nkv, self.d,
                            self.dtype)
-        attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
-                                         self.nkv, self.d, self.window, self.scale)
+        page_size = binding.cache.shape[3] // self.d
+        if ops.attention_mfma_takes(self.dtype, self.d, page_size):
+            tiles, nsplit = ctx.attention_tiles(self.nq // self.nkv, self.nkv)
+            attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv,
+                                          self.d, self.window, self.scale, nsplit)
+        else:
+            attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
+                                             self.nkv, self.d, self.window, self.scale)
         return self.o(attended)
 
     def _apply_other_positions(self, qkv, ctx):

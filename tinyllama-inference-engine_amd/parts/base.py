@@ -29,7 +29,7 @@ from ..ops import Product, as_product
 
 @dataclass(frozen=True)
 class KVCacheNeed:
-    """Pages of keys and values: [2, num_kv_heads, page_size, head_dim] per page.  `window`
+    """Pages of keys and values: [2, num_kv_heads, page_size * head_dim] per page.  `window`
     None: every key stays; else only the last `window` positions are ever read again."""
     num_kv_heads: int
     head_dim: int
@@ -47,7 +47,7 @@ class StateNeed:
 class Binding:
     """What the cache manager holds for one run of a layer."""
     group: int | None = None            # index of the page group (block table, slot map) in the step context
-    cache: torch.Tensor | None = None   # [pages, 2, nkv, page_size, d] of the run whose cache is read
+    cache: torch.Tensor | None = None   # [pages, 2, nkv, page_size * d] of the run whose cache is read
     writes: bool = True                 # this run owns the cache and writes the step's keys and values
     state: torch.Tensor | None = None   # [request slots, *shape] for a mixer with state of its own
 

@@ -4,7 +4,10 @@
 Which kernel runs is decided here and nowhere else:
   float32 activations            the true 32-bit kernel (plain FMAs, no matrix instruction)
   bfloat16, weight kept float32  the same kernel on widened values
-  bfloat16                       the tiled MFMA kernels when they take the sizes, else the plain one
+  bfloat16, at most 64 rows      the skinny MFMA kernel (W streamed once, split-K partial sums)
+  bfloat16, more rows            the library's product (as the reference uses a library for its
+                                 products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out
+  anything those refuse          the plain kernel
 """
 from __future__ import annotations
 
@@ -24,5 +27,16 @@ class Linear:
         self.out_features, self.in_features = self.weight.shape
 
     def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> Product:
+        """out_dtype: what a dense result is stored in (the skinny kernel's partial sums are float32
+        whatever it says)."""
         out_dtype = out_dtype or self.dtype
+        if ops.gemm_skinny_takes(x, self.weight):
+            return ops.gemm_skinny(x, self.weight, self.bias)
+        if x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
+            ops._device_tensor(x, "x", torch.bfloat16)
+            if x.dim() != 2 or x.shape[1] != self.in_features:
+                raise ops.invalid_shape(f"linear: x {list(x.shape)} does not fit weight {list(self.weight.shape)}")
+            if self.bias is not None:
+                return Product(torch.addmm(self.bias, x, self.weight.t()), 1)
+            return Product(torch.mm(x, self.weight.t()), 1)
         return ops.gemm_generic(x, self.weight, self.bias, out_dtype)
