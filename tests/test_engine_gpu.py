@@ -39,9 +39,10 @@ def plain_logits(setup, tokens):
     return setup["plain"][key]
 
 
-def new_engine(setup, dtype, max_tokens=512, page_size=16, max_requests=4):
+def new_engine(setup, dtype, max_tokens=512, page_size=16, max_requests=4, use_graphs=True):
     from tlie_amd import Engine
-    return Engine(setup["folder"], dtype=dtype, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests)
+    return Engine(setup["folder"], dtype=dtype, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests,
+                  use_graphs=use_graphs)
 
 
 def request_tokens(name, index, length):
@@ -203,6 +204,44 @@ def test_greedy_generation_through_the_entry_point(setups, name, dtype):
                 gap = (logits[want[same]] - logits[tokens[same]]).item()
                 assert 0 <= gap <= 2 * TOLERANCE[dtype] * logits.abs().max().item(), f"token {same} differs without a near tie"
     assert engine.cache.free_pages() == [engine.cache.num_pages]
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
+def test_recorded_decode_steps_replay_like_eager_ones(setups, name, dtype):
+    """Decode steps are recorded once per batch-size bucket into a HIP graph and replayed.  Every
+    replay is checked against an engine that launches the same steps one kernel at a time, with
+    prompt steps (never recorded) and synchronisations in between, batches that do not fill their
+    bucket, and a request that ends mid-way so that rows of the bucket become padding."""
+    setup = setups(name, dtype)
+    recorded, eager = new_engine(setup, dtype, max_tokens=1024, max_requests=8), \
+        new_engine(setup, dtype, max_tokens=1024, max_requests=8, use_graphs=False)
+    assert recorded.runner.use_graphs and not eager.runner.use_graphs
+    prompts = {f"g{i}": request_tokens(name, 70 + i, n) for i, n in enumerate((9, 33, 20))}
+    follow = {request: request_tokens(name, 80 + i, 40) for i, request in enumerate(prompts)}
+    a, b = Replayer(recorded), Replayer(eager)
+    for replay in (a, b):
+        replay.step([(request, tokens, [len(tokens) - 1]) for request, tokens in prompts.items()])
+    live = list(prompts)
+    for turn in range(24):
+        if turn == 9:
+            for replay in (a, b):                         # a prompt step between replays
+                replay.step([("late", follow["g0"][:13], [12])])
+            live.append("late")
+            follow["late"] = request_tokens(name, 90, 40)
+        if turn == 15:
+            for replay in (a, b):
+                replay.engine.finish("g1")
+            live.remove("g1")
+        items = [(request, [follow[request][turn]], [0]) for request in live]
+        a.step(items)
+        b.step(items)
+        torch.cuda.synchronize()
+    assert recorded.runner._graphs and all(graph.graph is not None for graph in recorded.runner._graphs.values())
+    assert set(a.rows) == set(b.rows)
+    keys = sorted(a.rows, key=str)
+    got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
+    bad = first_bad_row(got, want, CUT_TOLERANCE[dtype])
+    assert bad is None, f"replayed step differs from the eager one at {keys[bad]}"
 
 
 def error_code(stderr):

@@ -327,9 +327,16 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     table = torch.tensor([[0] * len(pages), pages], dtype=torch.int32, device=DEV)
     tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv)
     tiles[:, 0] = 1                                                            # the sequence is row 1 of the table
-    out = ops.attention_mfma(q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV), cache.to(DEV), table,
-                             torch.from_numpy(tiles).to(DEV), torch.tensor(token_list, dtype=torch.int32, device=DEV),
-                             nq, nkv, d, window, 1.0 / math.sqrt(d), nsplit)
+    split_len = ((tokens + nsplit - 1) // nsplit + 31) // 32 * 32
+    rows = q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV)
+    positions = torch.tensor(token_list, dtype=torch.int32, device=DEV)
+    out = ops.attention_mfma(rows, cache.to(DEV), table, torch.from_numpy(tiles).to(DEV), positions, nq, nkv, d, window,
+                             1.0 / math.sqrt(d), nsplit, split_len)
+    if len(token_list) == 1:
+        # the same step as a decode step: no work list, the kernel derives the tiles; the sequence must be row 0
+        decode = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
+                                    1.0 / math.sqrt(d), nsplit, split_len)
+        assert torch.equal(decode, out)
     return out.view(len(token_list), nq, d)
 
 
@@ -407,7 +414,7 @@ def test_attention_mfma_mixed_step():
     tiles = torch.from_numpy(ops.attention_tiles(seq_start, nq // nkv)).to(DEV)
     for nsplit in (1, 3):
         out = ops.attention_mfma(q_rows.contiguous().to(DEV), torch.cat(caches).to(DEV), table, tiles, positions, nq, nkv, d,
-                                 None, 1.0 / math.sqrt(d), nsplit).view(-1, nq, d)
+                                 None, 1.0 / math.sqrt(d), nsplit, 96).view(-1, nq, d)
         cursor = 0
         for index, (first, count) in enumerate(brings):
             want = plain_attention(rounded(qs[index], torch.bfloat16), rounded(ks[index], torch.bfloat16),

@@ -68,6 +68,24 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return total;
 }
 
+// The sum over `nsplit` partial results that lie `stride` elements apart, four loads in flight at a
+// time.  The order of the additions is fixed (four interleaved chains, then their sum), so the
+// result does not vary from run to run.
+template <typename D>
+__device__ __forceinline__ float sum_splits(const D* __restrict__ first, int nsplit, size_t stride) {
+  if (nsplit == 1) return to_float(first[0]);
+  float a = 0.f, b = 0.f, c = 0.f, d = 0.f;
+  int s = 0;
+  for (; s + 3 < nsplit; s += 4) {
+    a += to_float(first[(s + 0) * stride]);
+    b += to_float(first[(s + 1) * stride]);
+    c += to_float(first[(s + 2) * stride]);
+    d += to_float(first[(s + 3) * stride]);
+  }
+  for (; s < nsplit; ++s) a += to_float(first[s * stride]);
+  return (a + b) + (c + d);
+}
+
 // Error codes returned by the C entry points (0 = launched).
 constexpr int kOk = 0;
 constexpr int kBadArgument = -1;   // a size or dtype the kernel does not take

@@ -36,9 +36,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const D* __rest
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = res[i];
     if (delta) {
-      float d = 0.f;
-      for (int s = 0; s < nsplit; ++s) d += to_float(delta[s * split_stride + static_cast<size_t>(src) * hidden + i]);
-      v += d;
+      v += sum_splits(delta + static_cast<size_t>(src) * hidden + i, nsplit, split_stride);
       if (!rows) res[i] = v;
     }
     row_cache[i] = v;
@@ -61,12 +59,9 @@ __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_
   for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
        index += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t t = index / inter, i = index % inter;
-    float g = 0.f, u = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      const D* base = gate_up + s * split_stride + t * 2 * inter;
-      g += to_float(base[i]);
-      u += to_float(base[inter + i]);
-    }
+    const D* base = gate_up + t * 2 * inter;
+    const float g = sum_splits(base + i, nsplit, split_stride);
+    const float u = sum_splits(base + inter + i, nsplit, split_stride);
     out[index] = from_float<O>((g / (1.f + expf(-g))) * u);
   }
 }
@@ -94,7 +89,7 @@ template <typename D, typename W, typename O>
 static int launch_add_rmsnorm(float* residual, const void* delta, int nsplit, size_t split_stride,
                               const void* weight, float eps, void* out,
                               const int* rows, int num_rows, int hidden, hipStream_t stream) {
-  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+  const int threads = hidden >= 2048 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
   const size_t lds = (static_cast<size_t>(hidden) + 16) * sizeof(float);
   if (lds > 160 * 1024) return kBadArgument;
   hipLaunchKernelGGL((add_rmsnorm_kernel<D, W, O>), dim3(num_rows), dim3(threads), lds, stream, residual,

@@ -6,6 +6,9 @@
 // (kernels.cu:137-145) then copies the rotated key and the value to the cache row of the
 // position.  Here all tokens of a step go in one launch, positions come from an array, the
 // frequencies from a table made once per model, and the cache row is found through the slot map.
+// A block serves a few heads of one token: it first forms the token's d/2 sines and cosines once
+// (not once per head), then every thread sums its element's partial results, trades it with its
+// rotation partner through LDS, and writes q or the cache.
 #include "common.h"
 
 namespace tlie {
@@ -15,59 +18,54 @@ namespace tlie {
 // values at index 1 transposed, [dim][row] (the attention kernels read 4 consecutive rows of one dim).
 // slot_map[t] = page * page_size + row of token t, or -1: nothing is written for that token.
 // rot_dim <= d, even: dimensions from rot_dim on are copied unrotated.  inv_freq may be null
-// (no rotation at all).
+// (no rotation at all).  blockDim.x = heads_per_block * d; grid = (tokens, ceil(heads / heads_per_block)).
 template <typename D, typename A>
 __global__ void rope_cache_kernel(const D* __restrict__ qkv, int nsplit, size_t split_stride,
                                   const int* __restrict__ positions, const int* __restrict__ slot_map,
                                   const float* __restrict__ inv_freq, int rot_dim, A* __restrict__ q_out,
                                   A* __restrict__ cache, int nq, int nkv, int d, int page_size) {
+  extern __shared__ float lds[];
+  float* cosines = lds;                  // rot_dim / 2
+  float* sines = cosines + rot_dim / 2;  // rot_dim / 2
+  float* values = sines + rot_dim / 2;   // blockDim.x
   const int t = blockIdx.x;
-  const int width = (nq + 2 * nkv) * d;
-  const D* row = qkv + static_cast<size_t>(t) * width;
-  const float pos = static_cast<float>(positions[t]);
-  const int slot = slot_map[t];
+  const int heads = nq + 2 * nkv;
+  const int width = heads * d;
   const int half = rot_dim / 2;
-  const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * d;
-  A* cache_row = nullptr;
-  if (slot >= 0) cache_row = cache + static_cast<size_t>(slot / page_size) * page_stride + static_cast<size_t>(slot % page_size) * d;
-  const size_t head_stride = static_cast<size_t>(page_size) * d;
-
-  auto value = [&](int column) {
-    float v = 0.f;
-    for (int s = 0; s < nsplit; ++s) v += to_float(row[s * split_stride + column]);
-    return v;
-  };
-
-  // q and k heads: one work item per (head, i) with i < d/2 covers elements i and i + d/2 when
-  // both are unrotated, or the rotated pair (i, i + half) when i < half.
-  const int rotated_heads = nq + nkv;
-  const int items = rotated_heads * d;
-  for (int item = threadIdx.x; item < items; item += blockDim.x) {
-    const int head = item / d, e = item % d;
-    float result;
-    if (inv_freq != nullptr && e < rot_dim) {
-      const int i = e < half ? e : e - half;
-      const float angle = pos * inv_freq[i];
-      float sine, cosine;
-      sincosf(angle, &sine, &cosine);
-      const float first = value(head * d + i), second = value(head * d + i + half);
-      result = e < half ? first * cosine - second * sine : second * cosine + first * sine;
+  if (inv_freq != nullptr) {
+    const float pos = static_cast<float>(positions[t]);
+    for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
+  }
+  const int local_head = threadIdx.x / d, e = threadIdx.x % d;
+  const int head = blockIdx.y * (blockDim.x / d) + local_head;
+  const bool live = head < heads;
+  float mine = 0.f;
+  if (live) mine = sum_splits(qkv + static_cast<size_t>(t) * width + head * d + e, nsplit, split_stride);
+  values[threadIdx.x] = mine;
+  __syncthreads();
+  if (!live) return;
+  float result = mine;
+  if (inv_freq != nullptr && head < nq + nkv && e < rot_dim) {
+    if (e < half) {
+      result = mine * cosines[e] - values[threadIdx.x + half] * sines[e];
     } else {
-      result = value(head * d + e);
-    }
-    if (head < nq) {
-      q_out[static_cast<size_t>(t) * nq * d + head * d + e] = from_float<A>(result);
-    } else if (cache_row) {
-      cache_row[(head - nq) * head_stride + e] = from_float<A>(result);
+      result = mine * cosines[e - half] + values[threadIdx.x - half] * sines[e - half];
     }
   }
-  if (slot >= 0) {
-    A* v_page = cache + static_cast<size_t>(slot / page_size) * page_stride + static_cast<size_t>(nkv) * head_stride +
-                slot % page_size;
-    for (int item = threadIdx.x; item < nkv * d; item += blockDim.x) {
-      const int head = item / d, e = item % d;
-      v_page[head * head_stride + static_cast<size_t>(e) * page_size] = from_float<A>(value((nq + nkv + head) * d + e));
-    }
+  if (head < nq) {
+    q_out[static_cast<size_t>(t) * nq * d + head * d + e] = from_float<A>(result);
+    return;
+  }
+  const int slot = slot_map[t];
+  if (slot < 0) return;
+  const size_t head_stride = static_cast<size_t>(page_size) * d;
+  A* page = cache + static_cast<size_t>(slot / page_size) * 2 * nkv * head_stride;
+  const int row = slot % page_size;
+  if (head < nq + nkv) {
+    page[(head - nq) * head_stride + static_cast<size_t>(row) * d + e] = from_float<A>(result);
+  } else {
+    // value head (head - nq - nkv) lies after the nkv key heads: at head offset (head - nq), transposed
+    page[(head - nq) * head_stride + static_cast<size_t>(e) * page_size + row] = from_float<A>(result);
   }
 }
 
@@ -79,13 +77,20 @@ extern "C" int tlie_rope_cache(const void* qkv, int in_dtype, int nsplit, long l
                                const int* positions, const int* slot_map, const float* inv_freq, int rot_dim,
                                void* q_out, void* cache, int act_dtype, int tokens, int nq, int nkv, int d,
                                int page_size, void* stream) {
-  if (tokens <= 0 || nq <= 0 || nkv <= 0 || d <= 0 || page_size <= 0 || nsplit < 1) return kBadArgument;
+  if (tokens <= 0 || nq <= 0 || nkv <= 0 || d <= 0 || d > 1024 || page_size <= 0 || nsplit < 1) return kBadArgument;
   if (rot_dim < 0 || rot_dim > d || rot_dim % 2 != 0) return kBadArgument;
-  const int threads = (nq + nkv) * d >= 1024 ? 256 : 64;
+  const int heads = nq + 2 * nkv;
+  int heads_per_block = 256 / d;
+  if (heads_per_block < 1) heads_per_block = 1;
+  if (heads_per_block > heads) heads_per_block = heads;
+  const int threads = heads_per_block * d;
+  const dim3 grid(tokens, (heads + heads_per_block - 1) / heads_per_block);
+  if (grid.y > 65535) return kBadArgument;
+  const size_t lds = (static_cast<size_t>(rot_dim) + threads) * sizeof(float);
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(DC, D, AC, A)                                                                              \
   if (in_dtype == DC && act_dtype == AC) {                                                                   \
-    hipLaunchKernelGGL((rope_cache_kernel<D, A>), dim3(tokens), dim3(threads), 0, s, (const D*)qkv, nsplit,   \
+    hipLaunchKernelGGL((rope_cache_kernel<D, A>), grid, dim3(threads), lds, s, (const D*)qkv, nsplit,         \
                        (size_t)split_stride, positions, slot_map, inv_freq, rot_dim, (A*)q_out, (A*)cache, nq, \
                        nkv, d, page_size);                                                                   \
     return launch_status();                                                                                  \

@@ -39,7 +39,7 @@ def parse_dtype(name) -> torch.dtype:
 class Engine:
     def __init__(self, model_dir: str | None, dtype="bfloat16", max_tokens: int = 4096, page_size: int = 16,
                  max_requests: int = 64, device: str = "cuda:0", config: dict | None = None,
-                 random_seed: int | None = None):
+                 random_seed: int | None = None, use_graphs: bool = True):
         """max_tokens: how many positions the cache pools hold in all (rounded up to whole
         pages); max_requests: how many requests can be live at once.
 
@@ -67,7 +67,7 @@ class Engine:
         num_pages = (max_tokens + page_size - 1) // page_size
         self.cache = CacheManager(self.model.run_needs(), page_size, num_pages, max_requests, self.dtype, self.device,
                                   max_positions=self.spec.max_positions)
-        self.runner = ModelRunner(self.model, self.cache)
+        self.runner = ModelRunner(self.model, self.cache, use_graphs=use_graphs)
 
     # ---- the step function and what goes with it --------------------------------------------------
     def admit(self, request: Hashable) -> int:

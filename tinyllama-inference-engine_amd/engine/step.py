@@ -57,25 +57,40 @@ class StepContext:
     _tiles: dict = field(default_factory=dict)
 
     def attention_tiles(self, groups_per_kv: int, num_kv_heads: int):
-        """The tiled attention kernel's work list for this step (made once per group size), and
-        into how many parts each tile's key range is cut: as many as it takes to give a step of few
-        tiles about a thousand waves, each part at least 128 keys long."""
-        if groups_per_kv not in self._tiles:
-            from ..ops import attention_tiles
-            tiles = attention_tiles(self.host["seq_start"], groups_per_kv)
-            self._tiles[groups_per_kv] = torch.from_numpy(tiles).to(self.tokens.device)
-        tiles = self._tiles[groups_per_kv]
-        waves = tiles.shape[0] * num_kv_heads
-        nsplit = max(1, min((1024 + waves - 1) // waves, self.max_context // 128))
-        return tiles, nsplit
+        """The tiled attention kernel's work list for this step (made once per group size; None
+        for a decode step, whose tiles the kernel derives itself), and how the keys are cut: into
+        as many parts as it takes to give a step of few tiles about a thousand waves, each part a
+        multiple of 32 positions and at least 64.  Returns (tiles, nsplit, split_len)."""
+        decode = self.max_new == 1 and self.num_seqs == self.num_tokens
+        if decode:
+            tiles, count = None, self.num_tokens * ((groups_per_kv + 15) // 16)
+        else:
+            if groups_per_kv not in self._tiles:
+                from ..ops import attention_tiles
+                tiles = attention_tiles(self.host["seq_start"], groups_per_kv)
+                self._tiles[groups_per_kv] = torch.from_numpy(tiles).to(self.tokens.device)
+            tiles = self._tiles[groups_per_kv]
+            count = tiles.shape[0]
+        waves = count * num_kv_heads
+        nsplit = max(1, min((1024 + waves - 1) // waves, (self.max_context + 63) // 64))
+        if nsplit == 1:
+            return tiles, 1, 0
+        split_len = ((self.max_context + nsplit - 1) // nsplit + 31) // 32 * 32
+        nsplit = (self.max_context + split_len - 1) // split_len
+        return tiles, nsplit, split_len
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager):
+    def __init__(self, model, cache: CacheManager, use_graphs: bool = True):
         self.model = model
         self.cache = cache
         self.device = model.device
         self.vocab_size = model.spec.vocab_size
+        # Decode steps are bound by launches, not by the kernels: a step of single tokens whose
+        # kernels are all this engine's own is captured once per batch-size bucket as a HIP graph
+        # and replayed.  Parts say whether they may be captured (`graph_safe`).
+        self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
+        self._graphs: dict[int, "DecodeGraph"] = {}
 
     # ---- checks and context ------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -114,11 +129,106 @@ class ModelRunner:
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         for request, count in wanted:
             self.cache.reserve(request, count)
-        ctx = self.build_context(entries)
-        logits = self.model.forward(ctx, self.cache.bindings)
+        if self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH and \
+                all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries):
+            bucket = DecodeGraph.bucket_of(len(entries))
+            if bucket not in self._graphs:
+                self._graphs[bucket] = DecodeGraph(self, bucket)
+            logits = self._graphs[bucket].run(entries)
+        else:
+            ctx = self.build_context(entries)
+            logits = self.model.forward(ctx, self.cache.bindings)
         for request, count in wanted:
             self.cache.commit(request, count)
         return logits
+
+
+class DecodeGraph:
+    """A decode step for up to `bucket` sequences, one token each, every token's logits wanted:
+    the step's arrays live at fixed addresses, the model's kernels are recorded once into a HIP
+    graph and replayed with new contents.  Rows beyond the step's sequences are padding: token 0
+    at position 0 of a sequence with no page written (slot -1), whose results are dropped.
+    How the attention kernel cuts the key range is fixed at capture (for the longest sequence the
+    cache can hold); each part computes its own bounds from the positions on the device."""
+    MAX_BATCH = 64          # the largest step whose products all run in this engine's own kernels
+
+    @staticmethod
+    def bucket_of(count: int) -> int:
+        bucket = 1
+        while bucket < count:
+            bucket *= 2
+        return bucket
+
+    def __init__(self, runner: "ModelRunner", bucket: int):
+        self.runner, self.bucket = runner, bucket
+        cache = runner.cache
+        longest = cache.max_positions or cache.num_pages * cache.page_size
+        self.widths = [max(1, (longest + cache.page_size - 1) // cache.page_size) for _ in cache.groups]
+        layout = [("tokens", (bucket,)), ("positions", (bucket,)), ("token_seq", (bucket,)), ("no_slots", (bucket,)),
+                  ("seq_start", (bucket + 1,)), ("seq_first_pos", (bucket,)), ("seq_len", (bucket,)), ("seq_slot", (bucket,)),
+                  ("want_rows", (bucket,))]
+        for group, width in enumerate(self.widths):
+            layout += [(f"block_table{group}", (bucket, width)), (f"slot_map{group}", (bucket,))]
+        total = sum(int(np.prod(shape)) for _, shape in layout)
+        self.pinned = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.device_flat = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        flat = self.pinned.numpy()
+        self.host, views, cursor = {}, {}, 0
+        for name, shape in layout:
+            size = int(np.prod(shape))
+            self.host[name] = flat[cursor:cursor + size].reshape(shape)
+            views[name] = self.device_flat[cursor:cursor + size].view(shape)
+            cursor += size
+        self.host["token_seq"][:] = np.arange(bucket)
+        self.host["seq_start"][:] = np.arange(bucket + 1)
+        self.host["want_rows"][:] = np.arange(bucket)
+        self.host["no_slots"][:] = -1
+        groups = [GroupView(views[f"block_table{group}"], views[f"slot_map{group}"], width)
+                  for group, width in enumerate(self.widths)]
+        self.ctx = StepContext(
+            num_tokens=bucket, num_seqs=bucket, num_wanted=bucket, max_new=1, max_context=longest, tokens=views["tokens"],
+            positions=views["positions"], token_seq=views["token_seq"], no_slots=views["no_slots"],
+            seq_start=views["seq_start"], seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"],
+            seq_slot=views["seq_slot"], want_rows=views["want_rows"], groups=groups, host=self.host)
+        self.graph = None
+        self.logits = None
+
+    def _fill(self, entries: Sequence[StepEntry]) -> None:
+        cache, host, count = self.runner.cache, self.host, len(entries)
+        for name in ("tokens", "positions", "seq_first_pos", "seq_slot"):
+            host[name][count:] = 0
+        host["seq_len"][count:] = 1
+        for row, entry in enumerate(entries):
+            position = cache.length(entry.request)
+            host["tokens"][row] = int(entry.tokens[0])
+            host["positions"][row] = host["seq_first_pos"][row] = position
+            host["seq_len"][row] = position + 1
+            host["seq_slot"][row] = cache.slot(entry.request)
+        for group in range(len(cache.groups)):
+            table, slots = host[f"block_table{group}"], host[f"slot_map{group}"]
+            table[count:] = 0
+            slots[count:] = -1
+            for row, entry in enumerate(entries):
+                pages = cache.page_list(entry.request, group)
+                table[row, :len(pages)] = [page if page != ABSENT else 0 for page in pages]
+                slots[row] = cache.rows(entry.request, group, int(host["positions"][row]), 1)[0]
+
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        runner = self.runner
+        self._fill(entries)
+        self.device_flat.copy_(self.pinned, non_blocking=True)
+        if self.graph is None:
+            # the first step of this size runs eagerly (its result is used, and it leaves the
+            # context's work lists made); the same launches are then recorded for the steps to come
+            logits = runner.model.forward(self.ctx, runner.cache.bindings)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self.logits = runner.model.forward(self.ctx, runner.cache.bindings)
+            self.graph = graph
+            return logits[:len(entries)]
+        self.graph.replay()
+        return self.logits[:len(entries)]
 
 
 def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> StepContext:

@@ -45,6 +45,12 @@ class DecoderModel:
         self.final_norm.load(weights, "model.norm.")
         self.head.load(weights, "")
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be recorded into a HIP graph: every part says so."""
+        parts = [self.embedding, self.final_norm, self.head, *self.blocks]
+        return all(getattr(part, "graph_safe", False) for part in parts)
+
     def run_needs(self) -> list[RunNeed]:
         needs = []
         for run in self.spec.runs:

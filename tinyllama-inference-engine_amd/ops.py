@@ -266,18 +266,23 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p:
 
 # ---- bfloat16 kernels on the matrix cores ---------------------------------------------------------
 SKINNY_MAX_ROWS = 64
-_SKINNY_WAVES = 2048          # waves a skinny product is cut into at least, when K allows
-
-
 def skinny_split_len(rows: int, out_features: int, in_features: int) -> int:
-    """How many k values one split takes: enough splits that the product fills the chip's 256 CUs
-    with several waves each, never fewer than 128 k values (two 64-wide steps) per split, and
-    fewer splits for more rows, whose partial sums cost traffic of their own."""
+    """How many k values one split takes.  Measured on the MI355X over the TinyLlama shapes: a
+    workgroup that streams 256 to 512 k values of its 64 rows is fastest at every batch size;
+    longer splits leave the 256 CUs with too few workgroups to hide the first load's latency,
+    shorter ones pay more in partial sums than they gain.  Matrices with many rows (the gated
+    feed-forward's first product, the output head) take the longer splits, and more rows of x
+    take longer ones still, because each partial sum is a write and a read of rows x outputs."""
     strips = (out_features + 15) // 16
-    target = _SKINNY_WAVES if rows <= 16 else (_SKINNY_WAVES // 2 if rows <= 32 else _SKINNY_WAVES // 4)
-    splits = max(1, min((target + strips - 1) // strips, in_features // 128))
-    length = (in_features + splits - 1) // splits
-    return max(64, (length + 63) // 64 * 64)
+    if rows > 16 and strips >= 1024:
+        length = 1024
+    elif strips >= 512:
+        length = 512
+    else:
+        length = 256
+    if in_features >= 4096:
+        length = max(length, 512)            # a long inner size would leave its consumer too many partial sums
+    return min(length, (in_features + 63) // 64 * 64)
 
 
 def gemm_skinny_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -326,27 +331,39 @@ def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> b
     return dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= 256 and page_size % 4 == 0
 
 
-def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor,
+def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor | None,
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
-                   scale: float, nsplit: int = 1) -> torch.Tensor:
+                   scale: float, nsplit: int = 1, split_len: int = 0) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
-    positions: every tile's sequence is a row of block_table, its tokens are rows of q).  nsplit > 1
-    cuts every tile's key range into that many parts that run side by side and are merged."""
+    positions: every tile's sequence is a row of block_table, its tokens are rows of q); None for
+    a decode step, in which token i is the one token of sequence i.  nsplit > 1 cuts the keys into
+    that many parts of split_len positions (a multiple of 32; nsplit * split_len must reach the
+    longest sequence) that run side by side and are merged."""
     _device_tensor(q, "q", torch.bfloat16)
     _device_tensor(cache, "cache", torch.bfloat16)
     _device_tensor(block_table, "block_table", torch.int32)
-    _device_tensor(tiles, "tiles", torch.int32)
     _device_tensor(positions, "positions", torch.int32)
     tokens = q.shape[0]
     if q.shape != (tokens, num_heads * head_dim):
         raise invalid_shape(f"attention: q {list(q.shape)} is not [tokens, nq * d]")
     page_size = _check_cache(cache, num_kv_heads, head_dim, "attention")
-    if block_table.dim() != 2 or positions.shape != (tokens,) or tiles.dim() != 2 or tiles.shape[1] != 4 or tiles.shape[0] == 0:
-        raise invalid_shape("attention: block_table must be [sequences, max_blocks], positions [tokens], tiles [n, 4]")
+    if block_table.dim() != 2 or positions.shape != (tokens,):
+        raise invalid_shape("attention: block_table must be [sequences, max_blocks], positions [tokens]")
     if num_heads % num_kv_heads != 0:
         raise invalid_shape("attention: the number of heads must be a multiple of the number of kv heads")
+    if tiles is not None:
+        _device_tensor(tiles, "tiles", torch.int32)
+        if tiles.dim() != 2 or tiles.shape[1] != 4 or tiles.shape[0] == 0:
+            raise invalid_shape("attention: tiles must be [n, 4]")
+        num_tiles = tiles.shape[0]
+    else:
+        if block_table.shape[0] < tokens:
+            raise invalid_shape("attention: a decode step needs a block table row per token")
+        num_tiles = tokens * ((num_heads // num_kv_heads + 15) // 16)
+    if nsplit > 1 and (split_len <= 0 or split_len % 32 != 0):
+        raise invalid_argument("attention: split_len must be a positive multiple of 32")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
         raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a multiple of 4 rows")
     out = torch.empty_like(q)
@@ -355,7 +372,7 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
         part_o = torch.empty((tokens * num_heads * nsplit, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((tokens * num_heads * nsplit, 2), dtype=torch.float32, device=q.device)
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
-                                         tiles.shape[0], _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
-                                         tokens, num_heads, num_kv_heads, head_dim, page_size,
+                                         num_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
+                                         split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
                                          int(window) if window else 0, ctypes.c_float(scale), _stream()), "attention_mfma")
     return out

@@ -61,6 +61,11 @@ class Attention(Mixer):
         self.o = Linear(weights[prefix + "o_proj.weight"], weights.get(prefix + "o_proj.bias") if self.bias else None,
                         self.dtype)
 
+    @property
+    def graph_safe(self) -> bool:
+        # a position encoding applied as tensors may do anything; a rotation table (or none) is fused
+        return self.position.rotary_table() is not None or type(self.position).apply_qk is PositionEncoding.apply_qk
+
     def cache_need(self):
         return KVCacheNeed(self.nkv, self.d, int(self.window) if self.window is not None else None)
 
@@ -76,9 +81,9 @@ class Attention(Mixer):
                            self.dtype)
         page_size = binding.cache.shape[3] // self.d
         if ops.attention_mfma_takes(self.dtype, self.d, page_size):
-            tiles, nsplit = ctx.attention_tiles(self.nq // self.nkv, self.nkv)
+            tiles, nsplit, split_len = ctx.attention_tiles(self.nq // self.nkv, self.nkv)
             attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv,
-                                          self.d, self.window, self.scale, nsplit)
+                                          self.d, self.window, self.scale, nsplit, split_len)
         else:
             attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
                                              self.nkv, self.d, self.window, self.scale)

@@ -53,6 +53,11 @@ class Binding:
 
 
 class Part:
+    # A part whose forward only launches kernels on the current stream, with sizes that depend on
+    # nothing but the number of tokens and sequences (no reading of the step's host arrays, no
+    # synchronisation), may be recorded into a HIP graph.  Parts say so themselves.
+    graph_safe = False
+
     def __init__(self, spec: PartSpec, dtype: torch.dtype, device):
         self.spec = spec
         self.dtype = dtype              # the activation type: float32 or bfloat16

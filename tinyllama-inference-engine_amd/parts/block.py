@@ -39,6 +39,11 @@ class PreNormBlock:
         for attribute, place in self._PLACES:
             getattr(self, attribute).load(weights, self.layer.prefix + place)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", False)
+                   for part in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward))
+
     def forward(self, residual, pending, ctx, binding):
         normed = self.mixer_norm.add_forward(residual, pending)
         mixed = self.mixer.forward(normed, ctx, binding)

@@ -17,6 +17,7 @@ from .linear import Linear
 
 @register("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    graph_safe = True
     NAME = "model.embed_tokens.weight"
 
     def __init__(self, spec: PartSpec, dtype, device):
@@ -36,6 +37,7 @@ class TokenEmbedding(Part):
 
 @register("head", "lm_head")
 class LMHead(Part):
+    graph_safe = True
     NAME = "lm_head.weight"
 
     def __init__(self, spec: PartSpec, dtype, device):

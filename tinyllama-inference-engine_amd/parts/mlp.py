@@ -17,6 +17,7 @@ from .linear import Linear
 class GatedMLP(FeedForward):
     """spec: hidden_size, intermediate_size, activation ("silu").
     Tensors: `<prefix>{gate,up,down}_proj.weight`."""
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)

@@ -14,6 +14,7 @@ from .base import Norm, as_product
 @register("norm", "rms_norm")
 class RMSNorm(Norm):
     """spec: size, eps.  Tensor: `<prefix>weight` [size]."""
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)

@@ -15,6 +15,7 @@ from .base import PositionEncoding
 @register("position_encoding", "rotary")
 class Rotary(PositionEncoding):
     """spec: head_dim, theta, optionally rot_dim (default head_dim: the whole head turns)."""
+    graph_safe = True
 
     def __init__(self, spec: PartSpec, dtype, device):
         super().__init__(spec, dtype, device)
@@ -36,3 +37,4 @@ class Rotary(PositionEncoding):
 @register("position_encoding", "none")
 class NoPositions(PositionEncoding):
     """No position encoding in the mixer (keys are cached as projected)."""
+    graph_safe = True
