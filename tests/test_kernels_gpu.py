@@ -311,10 +311,16 @@ def test_gemm_skinny_refuses():
         ops.gemm_skinny(torch.randn(2, 12, device=DEV).bfloat16(), torch.randn(8, 12, device=DEV).bfloat16(), None)   # K % 8
     with pytest.raises(EngineError):
         ops.gemm_skinny(torch.randn(2, 64, device=DEV), w, None)                              # float32
+    assert not ops.attention_mfma_takes(torch.bfloat16, 64, 8)          # pages below 16 rows go to the plain kernel
+    assert not ops.attention_mfma_takes(torch.bfloat16, 72, 16) and not ops.attention_mfma_takes(torch.float32, 64, 16)
+    with pytest.raises(EngineError):
+        ops.attention_mfma(torch.zeros(1, 64, device=DEV).bfloat16(), torch.zeros(2, 2, 1, 8 * 64, device=DEV).bfloat16(),
+                           torch.zeros(1, 1, dtype=torch.int32, device=DEV), None, torch.zeros(1, dtype=torch.int32, device=DEV),
+                           1, 1, 64, None, 0.125)
     assert not ops.gemm_skinny_takes(torch.randn(2, 12, device=DEV).bfloat16(), torch.randn(8, 12, device=DEV).bfloat16())
 
 
-def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0):
+def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0, col_tiles=None):
     """One sequence through the tiled kernel: q rows for the positions in token_list (default all)."""
     from tlie_amd import ops
     import numpy as np
@@ -325,13 +331,14 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     # the step brings a run of consecutive positions of the one sequence
     assert token_list == list(range(token_list[0], token_list[0] + len(token_list)))
     table = torch.tensor([[0] * len(pages), pages], dtype=torch.int32, device=DEV)
-    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv)
+    col_tiles = col_tiles or ops.attention_col_tiles(d)
+    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv, col_tiles)
     tiles[:, 0] = 1                                                            # the sequence is row 1 of the table
     split_len = ((tokens + nsplit - 1) // nsplit + 31) // 32 * 32
     rows = q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV)
     positions = torch.tensor(token_list, dtype=torch.int32, device=DEV)
     out = ops.attention_mfma(rows, cache.to(DEV), table, torch.from_numpy(tiles).to(DEV), positions, nq, nkv, d, window,
-                             1.0 / math.sqrt(d), nsplit, split_len)
+                             1.0 / math.sqrt(d), nsplit, split_len, col_tiles)
     if len(token_list) == 1:
         # the same step as a decode step: no work list, the kernel derives the tiles; the sequence must be row 0
         decode = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
@@ -345,10 +352,10 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     dict(tokens=77, nq=6, nkv=3, d=48, page=16),
     dict(tokens=300, nq=5, nkv=5, d=80, page=32),
     dict(tokens=700, nq=8, nkv=1, d=128, page=16),
-    dict(tokens=333, nq=4, nkv=2, d=16, page=8, window=37),
+    dict(tokens=333, nq=4, nkv=2, d=16, page=32, window=37),
     dict(tokens=130, nq=3, nkv=1, d=256, page=64),
     dict(tokens=200, nq=32, nkv=4, d=64, page=16),
-    dict(tokens=150, nq=40, nkv=2, d=32, page=4, window=50),          # 20 heads a group: more than one tile per token
+    dict(tokens=150, nq=40, nkv=2, d=32, page=16, window=50),         # 20 heads a group: more than one tile per token
     dict(tokens=97, nq=7, nkv=7, d=112, page=16),
 ])
 def test_attention_mfma(case):
@@ -359,6 +366,8 @@ def test_attention_mfma(case):
     want = plain_attention(rounded(q, torch.bfloat16), rounded(k, torch.bfloat16), rounded(v, torch.bfloat16), window=window)
     whole = run_attention_mfma(q, k, v, page, window, 1, shuffle_seed=tokens)
     assert rel_err(whole, want) < TOL["bfloat16"]
+    narrow = run_attention_mfma(q, k, v, page, window, 1, shuffle_seed=tokens, col_tiles=1)       # 16 columns a wave
+    assert rel_err(narrow, want) < TOL["bfloat16"]
     # the last token alone (a decode step), its key range cut in parts that are merged
     for nsplit in (1, 2, 5):
         last = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=tokens)
@@ -411,10 +420,10 @@ def test_attention_mfma_mixed_step():
     q_rows = torch.cat([qs[i][first:first + count] for i, (first, count) in enumerate(brings)]).bfloat16().reshape(-1, nq * d)
     positions = torch.tensor([p for first, count in brings for p in range(first, first + count)], dtype=torch.int32, device=DEV)
     seq_start = np.cumsum([0] + [count for _, count in brings])
-    tiles = torch.from_numpy(ops.attention_tiles(seq_start, nq // nkv)).to(DEV)
+    tiles = torch.from_numpy(ops.attention_tiles(seq_start, nq // nkv, 4)).to(DEV)
     for nsplit in (1, 3):
         out = ops.attention_mfma(q_rows.contiguous().to(DEV), torch.cat(caches).to(DEV), table, tiles, positions, nq, nkv, d,
-                                 None, 1.0 / math.sqrt(d), nsplit, 96).view(-1, nq, d)
+                                 None, 1.0 / math.sqrt(d), nsplit, 96, 4).view(-1, nq, d)
         cursor = 0
         for index, (first, count) in enumerate(brings):
             want = plain_attention(rounded(qs[index], torch.bfloat16), rounded(ks[index], torch.bfloat16),

@@ -16,7 +16,9 @@
 //    are a reduction over 4 registers and 4 lane groups, and the probabilities are already laid out
 //    as operand B of the second product, O^T = V^T . P^T.  Nothing passes through LDS.
 //  * Values are cached transposed ([dim][row in page]), so operand A of the second product, 4
-//    consecutive keys of one dim, is one 8-byte load.
+//    consecutive keys of one dim, is one 8-byte load.  Pages hold at least 16 rows, so the 16 keys
+//    of half a block share a page: page numbers are scalar loads and a lane's addresses are a
+//    scalar base plus a constant.
 //  * Keys are walked in blocks of 32 that start at multiples of 32 from position 0, with a running
 //    maximum and sum: the context length is unbounded and the order of the sums for a (sequence,
 //    position) does not depend on how the step was cut.
@@ -28,23 +30,46 @@
 //    three loads in a row.
 #include "common.h"
 
+#include <type_traits>
+
 namespace tlie {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+
 union Pack8 {
   uint4 u;
   uint2 h[2];
+  uint32_t w[4];
   uint16_t e[8];
   bf16x8 v;
 };
 
-__device__ __forceinline__ uint16_t float_to_bf16_bits(float v) {
-  // round to nearest even; the inputs here are finite probabilities in [0, 1]
-  uint32_t bits = __float_as_uint(v);
-  bits += 0x7fffu + ((bits >> 16) & 1u);
-  return static_cast<uint16_t>(bits >> 16);
+// Reductions over the four lane groups of a column (lanes l, l ^ 16, l ^ 32, l ^ 48) with the
+// gfx950 row and half swaps: v_permlane16_swap exchanges the odd 16-lane rows of one operand with
+// the even rows of the other, v_permlane32_swap the upper half with the lower; with both operands
+// the same value, the two results hold a lane's own value and its partner's.
+typedef __attribute__((__vector_size__(2 * sizeof(unsigned)))) unsigned uintx2;
+__device__ __forceinline__ float groups_max(float v) {
+  uintx2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float groups_sum(float v) {
+  uintx2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// two floats to two bfloat16 (round to nearest even) in one instruction, v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  const bf16x2 r = __builtin_convertvector((floatx2{lo, hi}), bf16x2);
+  return *reinterpret_cast<const uint32_t*>(&r);
 }
 
 // tiles[i] = (sequence row of the block table, index of the sequence's first token in this step,
@@ -52,68 +77,95 @@ __device__ __forceinline__ uint16_t float_to_bf16_bits(float v) {
 // column c of a sequence = (token c / G of its tokens in this step, head c % G of the group).
 // tiles == nullptr: a decode step, token i is the one token of sequence i; the tile index is
 // sequence * ceil(G / 16) + tile of the group.
-// DT = head_dim / 16.
-template <int DT>
+// DT = head_dim / 16.  CT = groups of 16 columns per wave: a tile has 16 * CT columns, and every
+// key and value the wave loads serves all of them (prompt portions take CT = 4, decode steps 1).
+template <int DT, int CT>
 __global__ void __launch_bounds__(64)
 attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache,
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nsplit, int split_len, int nq, int nkv, int page_size,
-                      int window, float scale) {
+                      int window, float scale_log2) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;                 // 32-wide k steps of the first product
-  const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
+  const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
   const int kvh = blockIdx.y, split = blockIdx.z;
+  // whether a lane's 8 dims of k step ks exist: always, unless the head size is an odd multiple of 16
+  auto has_dims = [&](int ks) { return DT % 2 == 0 || ks < KS - 1 || grp < 2; };
   const int G = nq / nkv;
   int seq, tok0, ntok, col0;
   if (tiles != nullptr) {
     const int4 tile = tiles[blockIdx.x];
     seq = tile.x, tok0 = tile.y, ntok = tile.z, col0 = tile.w;
   } else {
-    const int per_seq = (G + 15) / 16;
-    seq = tok0 = blockIdx.x / per_seq, ntok = 1, col0 = (blockIdx.x % per_seq) * 16;
+    const int per_seq = (G + 16 * CT - 1) / (16 * CT);
+    seq = tok0 = blockIdx.x / per_seq, ntok = 1, col0 = (blockIdx.x % per_seq) * 16 * CT;
   }
-  const int pos0 = positions[tok0];
+  // everything about the tile is the same for all lanes: keep it in scalar registers, so that the
+  // conditions on it below are branches of the wave and not masks over its lanes
+  seq = __builtin_amdgcn_readfirstlane(seq), tok0 = __builtin_amdgcn_readfirstlane(tok0);
+  ntok = __builtin_amdgcn_readfirstlane(ntok), col0 = __builtin_amdgcn_readfirstlane(col0);
+  const int pos0 = __builtin_amdgcn_readfirstlane(positions[tok0]);
   const int ncols = ntok * G;
-  const int c = col0 + col;
-  const bool valid_col = c < ncols;
-  const int tok = tok0 + (valid_col ? c / G : 0);
-  const int head = kvh * G + (valid_col ? c % G : 0);
-  const int pos_col = valid_col ? pos0 + c / G : -1;
-  const int lo_col = window > 0 ? max(0, pos_col - window + 1) : 0;
+  bool valid_col[CT];
+  int tok[CT], head[CT], pos_col[CT], lo_col[CT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = col0 + ct * 16 + col;
+    valid_col[ct] = c < ncols;
+    tok[ct] = tok0 + (valid_col[ct] ? c / G : 0);
+    head[ct] = kvh * G + (valid_col[ct] ? c % G : 0);
+    pos_col[ct] = valid_col[ct] ? pos0 + c / G : -1;
+    lo_col[ct] = window > 0 ? max(0, pos_col[ct] - window + 1) : 0;
+  }
 
   // the tile's key range, and this split's part of it
-  const int last_col = min(col0 + 15, ncols - 1);
+  const int last_col = min(col0 + 16 * CT - 1, ncols - 1);
   const int tile_hi = pos0 + last_col / G + 1;
   const int tile_lo = window > 0 ? max(0, pos0 + col0 / G - window + 1) : 0;
   const int split_lo = nsplit > 1 ? split * split_len : 0;
   const int range_lo = max(tile_lo, split_lo);
   const int range_hi = nsplit > 1 ? min(tile_hi, split_lo + split_len) : tile_hi;
-  const int key_limit = max_blocks * page_size - 1;      // the last position the block table has an entry for
 
+  // Pages hold a power of two of rows, at least 16, and blocks of 32 keys start at multiples of 32:
+  // each half of a block (16 keys) lies on one page, the same for every lane.  So the page numbers
+  // are scalars, and a lane's addresses are a scalar base plus an offset that never changes.
+  const int page_shift = 31 - __clz(page_size), page_mask = page_size - 1;
   const int* pages = block_table + static_cast<size_t>(seq) * max_blocks;
   const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * D;
   const uint16_t* k_base = cache + static_cast<size_t>(kvh) * page_size * D;
-  const uint16_t* v_base = cache + static_cast<size_t>(nkv) * page_size * D + static_cast<size_t>(kvh) * page_size * D;
+  const uint16_t* v_base = k_base + static_cast<size_t>(nkv) * page_size * D;
+  const int k_lane = col * D + grp * 8;                    // operand A of the first product: key `col`, dims grp*8..
+  const int v_lane = (col << page_shift) + grp * 4;        // operand A of the second: dim `col`, keys grp*4..
 
   // Q as operand B: lane (col, grp) holds dims ks*32 + grp*8 .. +8 of its column
-  Pack8 qreg[KS];
+  Pack8 qreg[CT][KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int dim = ks * 32 + grp * 8;
-    qreg[ks].u = make_uint4(0, 0, 0, 0);
-    if (valid_col && dim < D) qreg[ks].u = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(tok) * nq + head) * D + dim);
+  for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int dim = ks * 32 + grp * 8;
+      qreg[ct][ks].u = make_uint4(0, 0, 0, 0);
+      if (valid_col[ct] && has_dims(ks))
+        qreg[ct][ks].u = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(tok[ct]) * nq + head[ct]) * D + dim);
+    }
+
+  // The softmax runs in base 2: scores are scaled by scale * log2(e) and exponentiated with exp2
+  // (one instruction); the result is the same function of the scores.
+  float running_max[CT], running_sum[CT];
+  floatx4 o[CT][DT];
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    running_max[ct] = -INFINITY, running_sum[ct] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[ct][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  float running_max = -INFINITY, running_sum = 0.f;
-  floatx4 o[DT];
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  // A block of 32 keys in registers: operand A of the first product (2 tiles of 16 keys) and of the
-  // second (per 16 dims, 2 x 4 consecutive keys).  Rows outside the range are read all the same,
-  // from whatever page the block table names there (absent entries name page 0), and masked or
-  // zeroed when used; so the addresses do not depend on the sequence's length.
+  // A block of 32 keys in registers: operand A of the first product (2 halves of 16 keys) and of
+  // the second (per 16 dims, 2 x 4 consecutive keys).  Rows outside the range are read all the
+  // same, from whatever page the block table names there (absent entries name page 0; past the
+  // table, its last entry), and masked or zeroed when used; so the addresses do not depend on the
+  // sequence's length and a block can be fetched before its turn.
   struct KeyBlock {
     Pack8 k[2][KS];
     uint2 v[DT][2];
@@ -121,129 +173,178 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   auto load_block = [&](int kb, KeyBlock& block) {
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const int key = min(kb + t * 16 + col, key_limit);
-      const uint16_t* k_row = k_base + static_cast<size_t>(pages[key / page_size]) * page_stride +
-                              static_cast<size_t>(key % page_size) * D;
+      const int first = kb + t * 16;
+      const int page = __builtin_amdgcn_readfirstlane(pages[min(first >> page_shift, max_blocks - 1)]);
+      const uint16_t* k_half = k_base + static_cast<size_t>(page) * page_stride + (first & page_mask) * D;
+      const uint16_t* v_half = v_base + static_cast<size_t>(page) * page_stride + (first & page_mask);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int dim = ks * 32 + grp * 8;
-        block.k[t][ks].u = dim < D ? *reinterpret_cast<const uint4*>(k_row + dim) : make_uint4(0, 0, 0, 0);
-      }
-    }
-    // slot i < 4 of group grp is key kb + grp*4 + i, slot i >= 4 is key kb + 16 + grp*4 + (i - 4)
-    const int clamp_a = min(kb + grp * 4, key_limit & ~3);
-    const int clamp_b = min(kb + 16 + grp * 4, key_limit & ~3);
-    const uint16_t* v_a = v_base + static_cast<size_t>(pages[clamp_a / page_size]) * page_stride + clamp_a % page_size;
-    const uint16_t* v_b = v_base + static_cast<size_t>(pages[clamp_b / page_size]) * page_stride + clamp_b % page_size;
+      for (int ks = 0; ks < KS; ++ks)
+        block.k[t][ks].u = has_dims(ks) ? *reinterpret_cast<const uint4*>(k_half + k_lane + ks * 32) : make_uint4(0, 0, 0, 0);
+      // slot i < 4 of group grp is key kb + grp*4 + i, slot i >= 4 is key kb + 16 + grp*4 + (i - 4)
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      const size_t dim = dt * 16 + col;
-      block.v[dt][0] = *reinterpret_cast<const uint2*>(v_a + dim * page_size);
-      block.v[dt][1] = *reinterpret_cast<const uint2*>(v_b + dim * page_size);
+      for (int dt = 0; dt < DT; ++dt)
+        block.v[dt][t] = *reinterpret_cast<const uint2*>(v_half + v_lane + ((dt * 16) << page_shift));
     }
   };
 
-  // without a window the first block's place is known before the position is: (split_lo & ~31)
-  const int first_block = (window > 0 ? range_lo : split_lo) & ~31;
-  KeyBlock next;
-  load_block(first_block, next);
-  for (int kb = first_block; kb < range_hi; kb += 32) {
-    KeyBlock block = next;
-    if (kb + 32 < range_hi) load_block(kb + 32, next);     // in flight while this block is worked on
-    // ---- S^T = K . Q^T for 2 x 16 keys -------------------------------------------------------
-    floatx4 s[2];
+  // masked_tag: whether any key of the block is hidden from any column of the tile (the range's
+  // ends, the causal diagonal, the window's edge); the many blocks in between take the other copy
+  // of this code, which has no comparisons in it
+  auto work_block = [&](int kb, KeyBlock& block, auto masked_tag) {
+    constexpr bool kMasked = decltype(masked_tag)::value;
+    const bool ragged = kMasked && (kb < range_lo || kb + 32 > range_hi);
+    if (ragged) {
+      // rows outside the range may hold anything (another request's values, or none ever
+      // written): zero them, so that 0 * NaN cannot arise
+      const int key_a = kb + grp * 4, key_b = kb + 16 + grp * 4;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(block.k[t][ks].v, qreg[ks].v, s[t], 0, 0, 0);
-    }
-    // ---- mask, scale, running softmax: s[t][j] is key kb + t*16 + grp*4 + j of column `col` ------
-    float block_max = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int key = kb + t * 16 + grp * 4 + j;
-        const bool ok = key >= range_lo && key < range_hi && key <= pos_col && key >= lo_col;
-        s[t][j] = ok ? s[t][j] * scale : -INFINITY;
-        block_max = fmaxf(block_max, s[t][j]);
-      }
-    block_max = fmaxf(block_max, __shfl_xor(block_max, 16, 64));
-    block_max = fmaxf(block_max, __shfl_xor(block_max, 32, 64));
-    const float new_max = fmaxf(running_max, block_max);
-    float alpha = 1.f, block_sum = 0.f;
-    Pack8 p;
-    if (new_max == -INFINITY) {
-      p.u = make_uint4(0, 0, 0, 0);                    // nothing visible to this column yet
-    } else {
-      alpha = expf(running_max - new_max);             // 0 while running_max is -inf
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float e = expf(s[t][j] - new_max);     // 0 for masked keys
-          block_sum += e;
-          p.e[t * 4 + j] = float_to_bf16_bits(e);
-        }
-    }
-    block_sum += __shfl_xor(block_sum, 16, 64);
-    block_sum += __shfl_xor(block_sum, 32, 64);
-    running_sum = running_sum * alpha + block_sum;
-    running_max = new_max;
-
-    // ---- O^T = O^T * alpha + V^T . P^T ---------------------------------------------------------
-    const bool ragged = kb < range_lo || kb + 32 > range_hi;
-    const int key_a = kb + grp * 4, key_b = kb + 16 + grp * 4;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      Pack8 a;
-      a.h[0] = block.v[dt][0];
-      a.h[1] = block.v[dt][1];
-      if (ragged) {
-        // rows outside the range may hold anything (another request's values, or none ever
-        // written): zero them, so that 0 * NaN cannot arise
+      for (int dt = 0; dt < DT; ++dt) {
+        Pack8 a;
+        a.h[0] = block.v[dt][0];
+        a.h[1] = block.v[dt][1];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           if (key_a + i < range_lo || key_a + i >= range_hi) a.e[i] = 0;
           if (key_b + i < range_lo || key_b + i >= range_hi) a.e[4 + i] = 0;
         }
+        block.v[dt][0] = a.h[0];
+        block.v[dt][1] = a.h[1];
       }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) o[dt][j] *= alpha;
-      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, o[dt], 0, 0, 0);
     }
-  }
-
-  // o[dt][j] is dim dt*16 + grp*4 + j of column `col`
-  if (!valid_col) return;
-  if (nsplit == 1) {
-    const float inv = 1.f / running_sum;
-    uint16_t* o_row = out + (static_cast<size_t>(tok) * nq + head) * D;
+    // The steps below run over all the wave's column groups one step at a time, not one group at
+    // a time: the groups do not depend on each other, and a wave issues in order.
+    // ---- S^T = K . Q^T for 2 x 16 keys ---------------------------------------------------------
+    floatx4 s[CT][2];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        s[ct][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(block.k[t][ks].v, qreg[ct][ks].v, s[ct][t], 0, 0, 0);
+      }
+    // ---- mask, scale, maximum: s[ct][t][j] is key kb + t*16 + grp*4 + j of the column --------------
+    float block_max[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      block_max[ct] = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (kMasked) {
+            const int key = kb + t * 16 + grp * 4 + j;
+            const bool ok = key >= range_lo && key < range_hi && key <= pos_col[ct] && key >= lo_col[ct];
+            s[ct][t][j] = ok ? s[ct][t][j] * scale_log2 : -INFINITY;
+          } else {
+            s[ct][t][j] *= scale_log2;
+          }
+          block_max[ct] = fmaxf(block_max[ct], s[ct][t][j]);
+        }
+    }
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) block_max[ct] = groups_max(block_max[ct]);
+    // ---- running softmax: the column's four lane groups share the maximum, so each keeps the sum of
+    // its own keys and the groups' sums are added once, after the last block ------------------------
+    float alpha[CT];
+    Pack8 p[CT];
+    bool changed = false;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const float new_max = fmaxf(running_max[ct], block_max[ct]);
+      alpha[ct] = 1.f;
+      if (kMasked && new_max == -INFINITY) {
+        p[ct].u = make_uint4(0, 0, 0, 0);              // nothing visible to this column yet
+      } else {
+        alpha[ct] = __builtin_amdgcn_exp2f(running_max[ct] - new_max);      // 0 while the running maximum is -inf
+        float e[8];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) e[t * 4 + j] = __builtin_amdgcn_exp2f(s[ct][t][j] - new_max);   // 0 for masked keys
+        running_sum[ct] = running_sum[ct] * alpha[ct] + (((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7])));
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[ct].w[i] = pack_bf16(e[2 * i], e[2 * i + 1]);
+      }
+      running_max[ct] = new_max;
+      changed = changed || alpha[ct] != 1.f;
+    }
+    // ---- O^T = O^T * alpha + V^T . P^T -----------------------------------------------------------
+    const bool rescale = __builtin_amdgcn_ballot_w64(changed) != 0;      // rare once the maxima have settled
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
-      uint2 packed;
-      packed.x = static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[dt][0] * inv))) |
-                 (static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[dt][1] * inv))) << 16);
-      packed.y = static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[dt][2] * inv))) |
-                 (static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[dt][3] * inv))) << 16);
-      *reinterpret_cast<uint2*>(o_row + dt * 16 + grp * 4) = packed;
-    }
-  } else {
-    const size_t slot = (static_cast<size_t>(tok) * nq + head) * nsplit + split;
-    float* po = part_o + slot * D;
+      Pack8 a;
+      a.h[0] = block.v[dt][0];
+      a.h[1] = block.v[dt][1];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-      *reinterpret_cast<float4*>(po + dt * 16 + grp * 4) = make_float4(o[dt][0], o[dt][1], o[dt][2], o[dt][3]);
-    if (grp == 0) {
-      part_ml[slot * 2] = running_max;
-      part_ml[slot * 2 + 1] = running_sum;
+      for (int ct = 0; ct < CT; ++ct) {
+        if (rescale) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[ct][dt][j] *= alpha[ct];
+        }
+        o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p[ct].v, o[ct][dt], 0, 0, 0);
+      }
+    }
+  };
+
+  // Two blocks in turn: while one is worked on, the other is on its way.  Without a window the
+  // first block's place is known before the position is: split_lo & ~31.
+  const int first_block = (window > 0 ? range_lo : split_lo) & ~31;
+  // a block that every column of the tile sees whole: inside the range, below the first column's
+  // position, inside the last column's window
+  const int open_lo = max((range_lo + 31) & ~31, window > 0 ? tile_hi - window : 0);
+  const int open_hi = min(range_hi, pos0 + col0 / G + 1) & ~31;
+  auto work = [&](int kb, KeyBlock& block) {
+    if (kb >= open_lo && kb + 32 <= open_hi)
+      work_block(kb, block, std::false_type{});
+    else
+      work_block(kb, block, std::true_type{});
+  };
+  KeyBlock even, odd;
+  load_block(first_block, even);
+  for (int kb = first_block; kb < range_hi; kb += 64) {
+    load_block(kb + 32, odd);
+    work(kb, even);
+    if (kb + 32 >= range_hi) break;
+    load_block(kb + 64, even);
+    work(kb + 32, odd);
+  }
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) running_sum[ct] = groups_sum(running_sum[ct]);
+
+  // o[ct][dt][j] is dim dt*16 + grp*4 + j of the column; maxima and sums are in base 2
+#pragma unroll
+  for (int ct = 0; ct < CT; ++ct) {
+    if (!valid_col[ct]) continue;
+    if (nsplit == 1) {
+      const float inv = 1.f / running_sum[ct];
+      uint16_t* o_row = out + (static_cast<size_t>(tok[ct]) * nq + head[ct]) * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        uint2 packed;
+        packed.x = static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[ct][dt][0] * inv))) |
+                   (static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[ct][dt][1] * inv))) << 16);
+        packed.y = static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[ct][dt][2] * inv))) |
+                   (static_cast<uint32_t>(__bfloat16_as_ushort(__float2bfloat16(o[ct][dt][3] * inv))) << 16);
+        *reinterpret_cast<uint2*>(o_row + dt * 16 + grp * 4) = packed;
+      }
+    } else {
+      const size_t slot = (static_cast<size_t>(tok[ct]) * nq + head[ct]) * nsplit + split;
+      float* po = part_o + slot * D;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        *reinterpret_cast<float4*>(po + dt * 16 + grp * 4) =
+            make_float4(o[ct][dt][0], o[ct][dt][1], o[ct][dt][2], o[ct][dt][3]);
+      if (grp == 0) {
+        part_ml[slot * 2] = running_max[ct];
+        part_ml[slot * 2 + 1] = running_sum[ct];
+      }
     }
   }
 }
 
-// out[t][h][:] = sum_p w_p O_p / sum_p w_p l_p with w_p = exp(m_p - max m).  One wave per (token, head);
+// out[t][h][:] = sum_p w_p O_p / sum_p w_p l_p with w_p = 2^(m_p - max m) (the maxima are in base 2).  One wave per (token, head);
 // the weights are formed once, by the lanes, and kept in LDS.
 __global__ void __launch_bounds__(64)
 attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -258,7 +359,7 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   float total = 0.f;
   for (int p = lane; p < nsplit; p += 64) {
     const float m = ml[p * 2];
-    const float w = m == -INFINITY ? 0.f : expf(m - top);
+    const float w = m == -INFINITY ? 0.f : exp2f(m - top);
     weight[p] = w;
     total += w * ml[p * 2 + 1];
   }
@@ -278,13 +379,14 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   }
 }
 
-template <int DT>
+template <int DT, int CT>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
                             int split_len, int nq, int nkv, int page_size, int window, float scale, hipStream_t stream) {
-  hipLaunchKernelGGL(attention_mfma_kernel<DT>, dim3(num_tiles, nkv, nsplit), dim3(64), 0, stream, (const uint16_t*)q,
+  const float scale_log2 = scale * 1.4426950408889634f;
+  hipLaunchKernelGGL((attention_mfma_kernel<DT, CT>), dim3(num_tiles, nkv, nsplit), dim3(64), 0, stream, (const uint16_t*)q,
                      (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                     part_ml, nsplit, split_len, nq, nkv, page_size, window, scale);
+                     part_ml, nsplit, split_len, nq, nkv, page_size, window, scale_log2);
   return launch_status();
 }
 
@@ -293,31 +395,53 @@ static int launch_attention(const void* q, const void* cache, const int* block_t
 using namespace tlie;
 
 // q, out: bfloat16 [tokens, nq, d]; cache: bfloat16 [pages, 2, nkv, page_size * d] (keys [row][dim], values [dim][row]).
-// tiles: int32 [num_tiles, 4], or null for a decode step (then num_tiles = tokens * ceil(G / 16)).
+// tiles: int32 [num_tiles, 4] with 16 * col_tiles columns each, or null for a decode step (then
+// col_tiles = 1 and num_tiles = tokens * ceil(G / 16)).
 // part_o: float [tokens * nq * nsplit * d], part_ml: float [tokens * nq * nsplit * 2] (both only when nsplit > 1);
 // split_len: positions per part, a multiple of 32, nsplit * split_len >= the longest sequence.
-// d % 16 == 0, d <= 256, page_size % 4 == 0.
+// d % 16 == 0, d <= 256, page_size a power of two >= 16; col_tiles 1, or 4 for d <= 64, or 2 for d <= 128.
 extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
-                                   const void* tiles, int num_tiles, const int* positions, void* out, float* part_o,
-                                   float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv, int d,
-                                   int page_size, int window, float scale, void* stream) {
+                                   const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
+                                   float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
+                                   int d, int page_size, int window, float scale, void* stream) {
   if (num_tiles <= 0 || tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || d % 16 != 0 ||
-      page_size < 4 || page_size % 4 != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
+      page_size < 16 || (page_size & (page_size - 1)) != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
     return kBadArgument;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr || split_len <= 0 || split_len % 32 != 0)) return kBadArgument;
-  if (tiles == nullptr && num_tiles != tokens * ((nq / nkv + 15) / 16)) return kBadArgument;
+  if (col_tiles != 1 && !(col_tiles == 4 && d <= 64) && !(col_tiles == 2 && d <= 128)) return kBadArgument;
+  if (tiles == nullptr && (col_tiles != 1 || num_tiles != tokens * ((nq / nkv + 15) / 16))) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
   int status = kBadArgument;
-#define TLIE_CASE(DT)                                                                                                  \
-  case DT:                                                                                                             \
-    status = launch_attention<DT>(q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, \
-                                  nsplit, split_len, nq, nkv, page_size, window, scale, s);                            \
+#define TLIE_ARGS q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, nsplit, split_len, nq, \
+                  nkv, page_size, window, scale, s
+#define TLIE_CASE(DT)                                        \
+  case DT:                                                   \
+    status = launch_attention<DT, 1>(TLIE_ARGS);             \
     break;
-  switch (d / 16) {
-    TLIE_CASE(1) TLIE_CASE(2) TLIE_CASE(3) TLIE_CASE(4) TLIE_CASE(5) TLIE_CASE(6) TLIE_CASE(7) TLIE_CASE(8)
-    TLIE_CASE(9) TLIE_CASE(10) TLIE_CASE(11) TLIE_CASE(12) TLIE_CASE(13) TLIE_CASE(14) TLIE_CASE(15) TLIE_CASE(16)
+#define TLIE_CASE4(DT)                                       \
+  case DT:                                                   \
+    status = launch_attention<DT, 4>(TLIE_ARGS);             \
+    break;
+#define TLIE_CASE2(DT)                                       \
+  case DT:                                                   \
+    status = launch_attention<DT, 2>(TLIE_ARGS);             \
+    break;
+  if (col_tiles == 1) {
+    switch (d / 16) {
+      TLIE_CASE(1) TLIE_CASE(2) TLIE_CASE(3) TLIE_CASE(4) TLIE_CASE(5) TLIE_CASE(6) TLIE_CASE(7) TLIE_CASE(8)
+      TLIE_CASE(9) TLIE_CASE(10) TLIE_CASE(11) TLIE_CASE(12) TLIE_CASE(13) TLIE_CASE(14) TLIE_CASE(15) TLIE_CASE(16)
+    }
+  } else if (col_tiles == 4) {
+    switch (d / 16) { TLIE_CASE4(1) TLIE_CASE4(2) TLIE_CASE4(3) TLIE_CASE4(4) }
+  } else {
+    switch (d / 16) {
+      TLIE_CASE2(1) TLIE_CASE2(2) TLIE_CASE2(3) TLIE_CASE2(4) TLIE_CASE2(5) TLIE_CASE2(6) TLIE_CASE2(7) TLIE_CASE2(8)
+    }
   }
 #undef TLIE_CASE
+#undef TLIE_CASE2
+#undef TLIE_CASE4
+#undef TLIE_ARGS
   if (status != kOk || nsplit == 1) return status;
   hipLaunchKernelGGL(attention_merge_kernel, dim3(tokens * nq), dim3(64), nsplit * sizeof(float), s, part_o, part_ml,
                      (uint16_t*)out, nsplit, d);

@@ -26,13 +26,14 @@ union Pack16 {
   bf16x8 v;
 };
 
-constexpr int kSkinnyThreads = 256;          // 4 waves, 16 rows of W each
-constexpr int kSkinnyRowsPerBlock = 64;
+constexpr int kSkinnyThreads = 256;          // 4 waves
 constexpr int kSkinnyPad = 8;                // bf16 elements of padding per LDS row (16 bytes): rows fall on different banks
 
-// NT: tiles of 16 rows of x (M <= 16 * NT).  CHUNK: k values staged in LDS at a time.
+// NT: tiles of 16 rows of x (M <= 16 * NT).  RS: strips of 16 rows of W per wave (a block takes
+// 64 * RS rows): with more rows of x, more strips share each read of x from LDS and each staging of
+// x from global memory.  CHUNK: k values staged in LDS at a time.
 // split_len: k values per split (multiple of 64).  K % 8 == 0.
-template <int NT, int CHUNK>
+template <int NT, int RS, int CHUNK>
 __global__ void __launch_bounds__(kSkinnyThreads)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
                    float* __restrict__ y, int M, int N, int K, int split_len) {
@@ -42,26 +43,34 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int split = blockIdx.y;
   const int k_begin = split * split_len, k_end = min(K, k_begin + split_len);
-  const int strip_row = blockIdx.x * kSkinnyRowsPerBlock + wave * 16;
+  const int wave_row = (blockIdx.x * 4 + wave) * 16 * RS;
   const int group = lane >> 4;
-  const bool active = strip_row < N;
-  const int row = min(strip_row + (lane & 15), N - 1);
-  const uint16_t* w_row = w + static_cast<size_t>(row) * K;
-
-  floatx4 acc[NT];
+  const uint16_t* w_row[RS];
+  bool active[RS];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < RS; ++r) {
+    active[r] = wave_row + r * 16 < N;
+    w_row[r] = w + static_cast<size_t>(min(wave_row + r * 16 + (lane & 15), N - 1)) * K;
+  }
+
+  floatx4 acc[RS][NT];
+#pragma unroll
+  for (int r = 0; r < RS; ++r)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   for (int c0 = k_begin; c0 < k_end; c0 += CHUNK) {
     const int c1 = min(k_end, c0 + CHUNK);
     // this wave's part of W for the chunk: issued first, in flight while x is staged
-    Pack16 a[kSteps][2];
+    Pack16 a[RS][kSteps][2];
 #pragma unroll
-    for (int s = 0; s < kSteps; ++s) {
-      const int k = c0 + s * 64 + group * 16;
-      a[s][0].u = (active && k < c1) ? *reinterpret_cast<const uint4*>(w_row + k) : make_uint4(0, 0, 0, 0);
-      a[s][1].u = (active && k + 8 < c1) ? *reinterpret_cast<const uint4*>(w_row + k + 8) : make_uint4(0, 0, 0, 0);
-    }
+    for (int r = 0; r < RS; ++r)
+#pragma unroll
+      for (int s = 0; s < kSteps; ++s) {
+        const int k = c0 + s * 64 + group * 16;
+        a[r][s][0].u = (active[r] && k < c1) ? *reinterpret_cast<const uint4*>(w_row[r] + k) : make_uint4(0, 0, 0, 0);
+        a[r][s][1].u = (active[r] && k + 8 < c1) ? *reinterpret_cast<const uint4*>(w_row[r] + k + 8) : make_uint4(0, 0, 0, 0);
+      }
     __syncthreads();                         // the previous chunk's reads of xs are done
     constexpr int kVectors = CHUNK / 8;
     for (int i = threadIdx.x; i < NT * 16 * kVectors; i += kSkinnyThreads) {
@@ -81,31 +90,38 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
         Pack16 b0, b1;
         b0.u = *reinterpret_cast<const uint4*>(x_row);
         b1.u = *reinterpret_cast<const uint4*>(x_row + 8);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][0].v, b0.v, acc[t], 0, 0, 0);
-        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][1].v, b1.v, acc[t], 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < RS; ++r) {
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[r][s][0].v, b0.v, acc[r][t], 0, 0, 0);
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[r][s][1].v, b1.v, acc[r][t], 0, 0, 0);
+        }
       }
     }
   }
-  if (!active) return;
-  // acc[t][j] = y[token t*16 + (lane & 15)][strip_row + group*4 + j]
-  const int n0 = strip_row + group * 4;
-  float add[4] = {0.f, 0.f, 0.f, 0.f};
-  if (bias != nullptr && split == 0) {
+  // acc[r][t][j] = y[token t*16 + (lane & 15)][wave_row + r*16 + group*4 + j]
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (n0 + j < N) add[j] = bf16_bits_to_float(bias[n0 + j]);
-  }
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int token = t * 16 + (lane & 15);
-    if (token >= M) continue;
-    float* out = y + (static_cast<size_t>(split) * M + token) * N + n0;
-    if ((N & 3) == 0 && n0 + 3 < N) {
-      *reinterpret_cast<float4*>(out) = make_float4(acc[t][0] + add[0], acc[t][1] + add[1], acc[t][2] + add[2], acc[t][3] + add[3]);
-    } else {
+  for (int r = 0; r < RS; ++r) {
+    if (!active[r]) continue;
+    const int n0 = wave_row + r * 16 + group * 4;
+    float add[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias != nullptr && split == 0) {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if (n0 + j < N) out[j] = acc[t][j] + add[j];
+        if (n0 + j < N) add[j] = bf16_bits_to_float(bias[n0 + j]);
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int token = t * 16 + (lane & 15);
+      if (token >= M) continue;
+      float* out = y + (static_cast<size_t>(split) * M + token) * N + n0;
+      if ((N & 3) == 0 && n0 + 3 < N) {
+        *reinterpret_cast<float4*>(out) =
+            make_float4(acc[r][t][0] + add[0], acc[r][t][1] + add[1], acc[r][t][2] + add[2], acc[r][t][3] + add[3]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (n0 + j < N) out[j] = acc[r][t][j] + add[j];
+      }
     }
   }
 }
@@ -122,17 +138,18 @@ extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, 
   const int nsplit = (K + split_len - 1) / split_len;
   const int tiles = (M + 15) / 16;
   const int nt = tiles <= 1 ? 1 : (tiles == 2 ? 2 : 4);
-  const dim3 grid((N + kSkinnyRowsPerBlock - 1) / kSkinnyRowsPerBlock, nsplit);
+  const int rows_per_block = nt == 4 ? 128 : 64;
+  const dim3 grid((N + rows_per_block - 1) / rows_per_block, nsplit);
   if (grid.y > 65535) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
   if (nt == 1)
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
   else if (nt == 2)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
   else
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 256>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 256>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
   return launch_status();
 }

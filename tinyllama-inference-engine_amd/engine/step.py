@@ -56,28 +56,34 @@ class StepContext:
     host: dict                     # the same arrays as numpy, by name
     _tiles: dict = field(default_factory=dict)
 
-    def attention_tiles(self, groups_per_kv: int, num_kv_heads: int):
+    def attention_tiles(self, groups_per_kv: int, num_kv_heads: int, head_dim: int):
         """The tiled attention kernel's work list for this step (made once per group size; None
         for a decode step, whose tiles the kernel derives itself), and how the keys are cut: into
-        as many parts as it takes to give a step of few tiles about a thousand waves, each part a
-        multiple of 32 positions and at least 64.  Returns (tiles, nsplit, split_len)."""
+        as many parts as it takes to give a step of few tiles about a thousand waves (measured: at
+        batch 64 and 2048 positions 4 parts reach 5 TB/s, 16 parts 4 TB/s, and merging more than 16
+        costs more than it gains), each part a multiple of 32 positions and at least 64.
+        Returns (tiles, col_tiles, nsplit, split_len)."""
         decode = self.max_new == 1 and self.num_seqs == self.num_tokens
+        col_tiles = 1
         if decode:
             tiles, count = None, self.num_tokens * ((groups_per_kv + 15) // 16)
         else:
-            if groups_per_kv not in self._tiles:
-                from ..ops import attention_tiles
-                tiles = attention_tiles(self.host["seq_start"], groups_per_kv)
-                self._tiles[groups_per_kv] = torch.from_numpy(tiles).to(self.tokens.device)
-            tiles = self._tiles[groups_per_kv]
+            from ..ops import attention_col_tiles, attention_tiles
+            col_tiles = attention_col_tiles(head_dim)
+            if (groups_per_kv, col_tiles) not in self._tiles:
+                tiles = attention_tiles(self.host["seq_start"], groups_per_kv, col_tiles)
+                self._tiles[(groups_per_kv, col_tiles)] = torch.from_numpy(tiles).to(self.tokens.device)
+            tiles = self._tiles[(groups_per_kv, col_tiles)]
             count = tiles.shape[0]
         waves = count * num_kv_heads
-        nsplit = max(1, min((1024 + waves - 1) // waves, (self.max_context + 63) // 64))
+        # a step of prompt portions has tiles enough; cutting their keys would only add merging
+        target = 1024 if decode else 512
+        nsplit = max(1, min((target + waves - 1) // waves, 16, (self.max_context + 63) // 64))
         if nsplit == 1:
-            return tiles, 1, 0
+            return tiles, col_tiles, 1, 0
         split_len = ((self.max_context + nsplit - 1) // nsplit + 31) // 32 * 32
         nsplit = (self.max_context + split_len - 1) // split_len
-        return tiles, nsplit, split_len
+        return tiles, col_tiles, nsplit, split_len
 
 
 class ModelRunner:

@@ -313,34 +313,42 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None
     return Product(out, nsplit)
 
 
-def attention_tiles(seq_start, groups_per_kv: int):
+def attention_col_tiles(head_dim: int) -> int:
+    """How many groups of 16 columns a wave of the tiled attention kernel serves in a step that
+    brings prompt portions: as many as its registers hold for the head size."""
+    return 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
+
+
+def attention_tiles(seq_start, groups_per_kv: int, col_tiles: int = 1):
     """The work list of the tiled attention kernel for a step, on the host: for every sequence,
-    tiles of 16 columns, a column being a (token, query head of one group) pair.
+    tiles of 16 * col_tiles columns, a column being a (token, query head of one group) pair.
     seq_start: the step's cumulative token counts [S + 1].  Returns an int32 array [tiles, 4]:
     (sequence, its first token's index in the step, its number of tokens, the tile's first column)."""
     import numpy as np
     rows = []
     for seq in range(len(seq_start) - 1):
         first, count = int(seq_start[seq]), int(seq_start[seq + 1] - seq_start[seq])
-        for col0 in range(0, count * groups_per_kv, 16):
+        for col0 in range(0, count * groups_per_kv, 16 * col_tiles):
             rows.append((seq, first, count, col0))
     return np.asarray(rows, dtype=np.int32).reshape(-1, 4)
 
 
 def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
-    return dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= 256 and page_size % 4 == 0
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= 256 and page_size >= 16
+            and page_size & (page_size - 1) == 0)
 
 
 def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor | None,
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
-                   scale: float, nsplit: int = 1, split_len: int = 0) -> torch.Tensor:
+                   scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
     positions: every tile's sequence is a row of block_table, its tokens are rows of q); None for
     a decode step, in which token i is the one token of sequence i.  nsplit > 1 cuts the keys into
     that many parts of split_len positions (a multiple of 32; nsplit * split_len must reach the
-    longest sequence) that run side by side and are merged."""
+    longest sequence) that run side by side and are merged.  col_tiles: the value the tiles were
+    made with."""
     _device_tensor(q, "q", torch.bfloat16)
     _device_tensor(cache, "cache", torch.bfloat16)
     _device_tensor(block_table, "block_table", torch.int32)
@@ -358,21 +366,24 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
         if tiles.dim() != 2 or tiles.shape[1] != 4 or tiles.shape[0] == 0:
             raise invalid_shape("attention: tiles must be [n, 4]")
         num_tiles = tiles.shape[0]
+        if col_tiles not in (1, 2, 4) or col_tiles > attention_col_tiles(head_dim):
+            raise invalid_argument(f"attention: {col_tiles} column groups a wave do not fit head size {head_dim}")
     else:
+        col_tiles = 1
         if block_table.shape[0] < tokens:
             raise invalid_shape("attention: a decode step needs a block table row per token")
         num_tiles = tokens * ((num_heads // num_kv_heads + 15) // 16)
     if nsplit > 1 and (split_len <= 0 or split_len % 32 != 0):
         raise invalid_argument("attention: split_len must be a positive multiple of 32")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
-        raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a multiple of 4 rows")
+        raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a power of two of rows (at least 16)")
     out = torch.empty_like(q)
     part_o = part_ml = None
     if nsplit > 1:
         part_o = torch.empty((tokens * num_heads * nsplit, head_dim), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((tokens * num_heads * nsplit, 2), dtype=torch.float32, device=q.device)
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
-                                         num_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
+                                         num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
                                          split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
                                          int(window) if window else 0, ctypes.c_float(scale), _stream()), "attention_mfma")
     return out
