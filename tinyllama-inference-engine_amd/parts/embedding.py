@@ -56,4 +56,4 @@ class LMHead(Part):
         self.linear = Linear(matrix, None, self.dtype)
 
     def forward(self, normed: torch.Tensor) -> torch.Tensor:
-        return self.linear(normed, out_dtype=torch.float32).dense(torch.float32)
+        return self.linear(normed, out_dtype=torch.float32, whole=True).dense(torch.float32)

@@ -26,12 +26,14 @@ class Linear:
         self.dtype = dtype
         self.out_features, self.in_features = self.weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None) -> Product:
+    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None, whole: bool = False) -> Product:
         """out_dtype: what a dense result is stored in (the skinny kernel's partial sums are float32
-        whatever it says)."""
+        whatever it says).  whole: the caller has no kernel that adds partial sums up, so the
+        product must come as one array (the skinny kernel then does not split K)."""
         out_dtype = out_dtype or self.dtype
-        if ops.gemm_skinny_takes(x, self.weight):
-            return ops.gemm_skinny(x, self.weight, self.bias)
+        if ops.gemm_skinny_takes(x, self.weight) and (not whole or out_dtype == torch.float32):
+            split_len = (self.in_features + 63) // 64 * 64 if whole else None
+            return ops.gemm_skinny(x, self.weight, self.bias, split_len=split_len)
         if x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
             ops._device_tensor(x, "x", torch.bfloat16)
             if x.dim() != 2 or x.shape[1] != self.in_features:
