@@ -430,3 +430,90 @@ def test_attention_mfma_mixed_step():
                                    rounded(vs[index], torch.bfloat16))[first:first + count]
             assert rel_err(out[cursor:cursor + count], want) < TOL["bfloat16"], f"sequence {index}, nsplit {nsplit}"
             cursor += count
+
+
+# ---- at most 16 rows: products with the norm before and the gate or the residual add after ----------------
+
+def partial_sums_of_squares(rows, columns_per_part=16):
+    """[ceil(width / columns_per_part), 16]: per group of columns and per row the sum of squares, as the
+    kernels leave it."""
+    count, width = rows.shape
+    parts = (width + columns_per_part - 1) // columns_per_part
+    padded = torch.zeros(count, parts * columns_per_part, dtype=torch.float64)
+    padded[:, :width] = rows.double()
+    out = torch.zeros(parts, 16, dtype=torch.float64)
+    out[:, :count] = (padded.view(count, parts, columns_per_part) ** 2).sum(-1).T
+    return out
+
+
+@pytest.mark.parametrize("shape", [(1, 40, 64), (3, 177, 176), (8, 2560, 2048), (16, 100, 520), (5, 2048, 5632), (11, 50, 8),
+                                   (16, 11264, 2048), (2, 4100, 1000)])
+def test_gemm_rows(shape):
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(n + m)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    b = torch.randn(n).bfloat16()
+    want = plain_linear(x.double(), w.double(), b.double())
+    got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV)).dense()
+    assert got.dtype == torch.float32 and rel_err(got, want) < 5e-6
+    for waves in (4, 8, 16):
+        for rows_per_block in (8, 16):
+            got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), waves=waves, rows_per_block=rows_per_block).dense()
+            assert rel_err(got, want) < 5e-6, (waves, rows_per_block)
+    # the norm before the product, folded in: the product runs on residual * g, its rows are scaled
+    residual = torch.randn(m, k) * 3
+    g = (1 + 0.2 * torch.randn(k)).bfloat16()
+    eps = 1e-5
+    xg = (residual * g.float()).bfloat16()
+    scale = 1.0 / torch.sqrt((residual.double() ** 2).mean(-1, keepdim=True) + eps)
+    want = plain_linear(xg.double(), w.double()) * scale + b.double()
+    for columns in (16, 8):                       # the partial sums may come per 16 columns or per 8
+        normed = ops.NormedRows(xg.to(DEV), partial_sums_of_squares(residual, columns).float().to(DEV), eps)
+        got = ops.gemm_rows(normed, w.to(DEV), b.to(DEV)).dense()
+        assert rel_err(got, want) < 1e-5
+    # and it is the norm: against RMSNorm then product, within the rounding of the input to bfloat16
+    want_normed = plain_linear(plain_rms_norm(residual, g.double(), eps), w.double(), b.double())
+    assert rel_err(got, want_normed) < TOL["bfloat16"]
+    if n % 2 == 0:
+        # rows of W alternate gate and up
+        full = plain_linear(x.double(), w.double())
+        for rows_per_block in (8, 16):
+            act = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "silu", rows_per_block=rows_per_block)
+            assert act.shape == (m, n // 2) and rel_err(act, plain_silu_mul(full[:, 0::2], full[:, 1::2])) < TOL["bfloat16"]
+        # the same layout through the kernel that adds up partial sums
+        parts = ops.gemm_skinny(x.to(DEV), w.to(DEV), None, split_len=64)
+        assert rel_err(ops.silu_mul(parts, torch.bfloat16, interleaved=True), plain_silu_mul(full[:, 0::2], full[:, 1::2])) < TOL["bfloat16"]
+    # added into the residual, with the next norm's inputs
+    target = torch.randn(m, n)
+    next_g = (1 + 0.2 * torch.randn(n)).bfloat16()
+    for next_weight, rows_per_block in ((next_g, 16), (next_g.float(), 8)):
+        res_dev = target.clone().to(DEV)
+        updated = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), "residual", residual=res_dev,
+                                next_norm=(next_weight.to(DEV), 1e-6), rows_per_block=rows_per_block)
+        want_res = target.double() + plain_linear(x.double(), w.double(), b.double())
+        assert rel_err(res_dev, want_res) < 5e-6
+        assert rel_err(updated.normed.xg, want_res * next_g.double()) < TOL["bfloat16"]
+        assert rel_err(updated.normed.ssq[:, :m], partial_sums_of_squares(res_dev.cpu(), rows_per_block)[:, :m]) < 1e-5
+        assert updated.normed.eps == 1e-6
+    res_dev = target.clone().to(DEV)
+    plain_update = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "residual", residual=res_dev)
+    assert plain_update.normed is None and rel_err(res_dev, target.double() + plain_linear(x.double(), w.double())) < 5e-6
+
+
+def test_embed_rows_and_refusals():
+    from tlie_amd import EngineError, ops
+    table = torch.randn(301, 72).bfloat16().to(DEV)
+    g = (1 + 0.2 * torch.randn(72)).bfloat16().to(DEV)
+    tokens = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
+    residual, normed = ops.embed_rows(tokens, table, (g, 1e-5))
+    rows = table.float().cpu()[tokens.long().cpu()]
+    assert torch.equal(residual.cpu(), rows)
+    assert rel_err(normed.xg, rows.double() * g.double().cpu()) < TOL["bfloat16"]
+    assert rel_err(normed.ssq[:, :5], partial_sums_of_squares(rows)[:, :5]) < 1e-5
+    with pytest.raises(EngineError):
+        ops.gemm_rows(torch.randn(17, 64, device=DEV).bfloat16(), torch.randn(8, 64, device=DEV).bfloat16(), None)
+    with pytest.raises(EngineError):
+        ops.gemm_rows(torch.randn(2, 64, device=DEV).bfloat16(), torch.randn(7, 64, device=DEV).bfloat16(), None, "silu")
+    assert not ops.gemm_rows_takes(4, torch.randn(8, 12, device=DEV).bfloat16(), torch.bfloat16)

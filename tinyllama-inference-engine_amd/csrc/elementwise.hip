@@ -50,18 +50,19 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const D* __rest
   }
 }
 
-// ---- act[t, i] = silu(gate[t, i]) * up[t, i]; gate_up is [rows, 2 * inter] = [gate | up] -------
+// ---- act[t, i] = silu(gate[t, i]) * up[t, i]; gate_up is [rows, 2 * inter], either [gate | up] or,
+// interleaved, g0 u0 g1 u1 ... (the layout the gated product of few rows wants of its weight) -------
 // reference: (g / (1 + exp(-g))) * u in float (src/cuda/kernels.cu:198-206)
 template <typename D, typename O>
 __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_t split_stride,
-                                O* __restrict__ out, int rows, int inter) {
+                                O* __restrict__ out, int rows, int inter, int interleaved) {
   const size_t total = static_cast<size_t>(rows) * inter;
   for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
        index += static_cast<size_t>(gridDim.x) * blockDim.x) {
     const size_t t = index / inter, i = index % inter;
     const D* base = gate_up + t * 2 * inter;
-    const float g = sum_splits(base + i, nsplit, split_stride);
-    const float u = sum_splits(base + inter + i, nsplit, split_stride);
+    const float g = sum_splits(base + (interleaved ? 2 * i : i), nsplit, split_stride);
+    const float u = sum_splits(base + (interleaved ? 2 * i + 1 : inter + i), nsplit, split_stride);
     out[index] = from_float<O>((g / (1.f + expf(-g))) * u);
   }
 }
@@ -120,7 +121,7 @@ extern "C" int tlie_add_rmsnorm(float* residual, const void* delta, int delta_dt
 }
 
 extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long long split_stride, void* out,
-                             int out_dtype, int rows, int inter, void* stream) {
+                             int out_dtype, int rows, int inter, int interleaved, void* stream) {
   if (rows <= 0 || inter <= 0 || nsplit < 1) return kBadArgument;
   const size_t total = static_cast<size_t>(rows) * inter;
   const int threads = 256;
@@ -128,13 +129,13 @@ extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long
   hipStream_t s = (hipStream_t)stream;
   if (in_dtype == kF32 && out_dtype == kF32)
     hipLaunchKernelGGL((silu_mul_kernel<float, float>), dim3(blocks), dim3(threads), 0, s, (const float*)gate_up, nsplit,
-                       (size_t)split_stride, (float*)out, rows, inter);
+                       (size_t)split_stride, (float*)out, rows, inter, interleaved);
   else if (in_dtype == kF32 && out_dtype == kBF16)
     hipLaunchKernelGGL((silu_mul_kernel<float, bf16>), dim3(blocks), dim3(threads), 0, s, (const float*)gate_up, nsplit,
-                       (size_t)split_stride, (bf16*)out, rows, inter);
+                       (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
   else if (in_dtype == kBF16 && out_dtype == kBF16)
     hipLaunchKernelGGL((silu_mul_kernel<bf16, bf16>), dim3(blocks), dim3(threads), 0, s, (const bf16*)gate_up, nsplit,
-                       (size_t)split_stride, (bf16*)out, rows, inter);
+                       (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
   else
     return kBadArgument;
   return launch_status();

@@ -1,0 +1,264 @@
+// y = x . W^T for at most 16 rows of x (decoding at small batch), bfloat16 on the matrix cores, with
+// what stands before and after the product in the layer folded into it, so that a decode step
+// needs fewer kernels: the scale of the RMSNorm before it, the bias, and then either the SiLU gate,
+// or the add into the residual together with the next norm's inputs.
+//
+// reference: one token's layer in the reference is 15 launches (2 norms, 7 products, rotation,
+// cache write, attention, SiLU, 2 adds; src/cuda/model.cu:406-475).  On this machine a dependent
+// launch costs 2 to 3 us even inside a replayed graph, as much as streaming a whole projection
+// matrix, so the count of launches decides the speed of decoding.  Finishing a split-K sum across
+// workgroups costs about as much (the L2 caches of the chip's eight dies do not see each other's
+// lines, so the parts have to travel through memory); here the sum stays inside a workgroup.
+//
+// A workgroup owns one MFMA strip of W's rows (16, or 8 when W has too few rows to give every CU
+// a workgroup) and all of K: its 4, 8 or 16 waves take a part of K each, read W and x straight
+// into the MFMA operands (no LDS staging: a wave's part of x is as small as its part of W), and
+// add their results up through LDS in a fixed order.  Because the workgroup then holds complete
+// sums, the epilogue can finish the layer's arithmetic:
+//
+//   * row scale: y[m, :] *= rsqrt(ssq[m] / width + eps).  RMSNorm(h) * g . W^T equals
+//     r * ((h * g) . W^T) with r the row's scalar, so the product runs on bfloat16(h * g) (stored
+//     by the previous epilogue, see below) and r is applied here; ssq[m] is the sum of the partial
+//     sums of squares that the previous epilogue left per 16 columns.
+//   * store: float32 [M, N] (qkv for the rotation kernel; logits).
+//   * SiLU gate: W's rows alternate gate and up (g0, u0, g1, u1, ...); out[m, i] = silu(g) * u,
+//     bfloat16 [M, N / 2].
+//   * residual: residual[m, n] += y (float32, in place: every element has one owner), and for the
+//     norm that reads the residual next: xg[m, n] = bfloat16(residual * g_next[n]) and the partial
+//     sums of squares per row and 16 columns.
+#include "common.h"
+
+namespace tlie {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+union RowPack {
+  uint4 u;
+  bf16x8 v;
+};
+
+constexpr int kEpilogueStore = 0, kEpilogueSilu = 1, kEpilogueResidual = 2;
+
+struct RowsArgs {
+  const uint16_t* x;          // [M, K] bfloat16
+  const uint16_t* w;          // [N, K] bfloat16
+  const uint16_t* bias;       // [N] or null
+  int M, N, K, k_per_wave;    // k_per_wave: multiple of 64
+  int rows_per_block;         // 16 or 8
+  // row scale (null: none)
+  const float* ssq_in;        // [strips_in, 16] partial sums of squares of the normed input's rows, over any split of its columns
+  int strips_in;
+  float inv_width, eps;       // 1 / width of the normed input
+  // outputs
+  float* y;                   // store: [M, N]
+  uint16_t* act;              // SiLU: [M, N / 2]
+  float* residual;            // residual: [M, N], updated in place
+  const uint16_t* next_weight;  // residual: [N] bfloat16 weight of the next norm, or null
+  const float* next_weight_f32; // the same when that weight is kept in float32
+  uint16_t* xg;               // residual: [M, N] bfloat16(residual * next weight), or null
+  float* ssq_out;             // residual: [ceil(N / rows_per_block), 16], or null
+};
+
+// WAVES: 4, 8 or 16 waves share K (more waves for a long K or few strips, fewer when the strips
+// alone fill the chip: every wave costs a dispatch).
+template <int EPILOGUE, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_rows_kernel(const RowsArgs a) {
+  __shared__ float partial[WAVES][64][4];           // each wave's 16 x 16 sums
+  __shared__ float scale_part[WAVES * 4][16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int block_row = blockIdx.x * a.rows_per_block;
+  const bool row_live = col < a.rows_per_block && block_row + col < a.N;      // with 8 rows a block, half the strip is idle
+  const int k_begin = wave * a.k_per_wave, k_end = min(a.K, k_begin + a.k_per_wave);
+  const uint16_t* w_row = a.w + static_cast<size_t>(min(block_row + col, a.N - 1)) * a.K;
+  const uint16_t* x_row = a.x + static_cast<size_t>(min(col, a.M - 1)) * a.K;
+  const bool token_live = col < a.M;
+
+  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = k_begin; k0 < k_end; k0 += 512) {
+    // 512 k of W at once (16 loads of 16 bytes per lane in flight: the weights come from HBM and a
+    // wave has nothing else to do meanwhile); x, which comes from the caches, in two halves
+    RowPack wa[8][2];
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int k = k0 + s * 64 + grp * 16;
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        wa[s][h].u = row_live && k + h * 8 < k_end ? *reinterpret_cast<const uint4*>(w_row + k + h * 8) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      if (k0 + half * 256 >= k_end) break;
+      RowPack xb[4][2];
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const int k = k0 + (half * 4 + s) * 64 + grp * 16;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          xb[s][h].u = k + h * 8 < k_end && token_live ? *reinterpret_cast<const uint4*>(x_row + k + h * 8)
+                                                       : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[half * 4 + s][0].v, xb[s][0].v, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[half * 4 + s][1].v, xb[s][1].v, acc, 0, 0, 0);
+      }
+    }
+  }
+  // acc[j] = sum over this wave's k of W[block_row + grp*4 + j][k] * x[col][k]
+#pragma unroll
+  for (int j = 0; j < 4; ++j) partial[wave][lane][j] = acc[j];
+  if (a.ssq_in != nullptr) {
+    // the (wave, group) pairs share the strips of the previous product; token = col
+    const int part = wave * 4 + grp;
+    float sum = 0.f;
+    for (int s = part; s < a.strips_in; s += WAVES * 4) sum += a.ssq_in[s * 16 + col];
+    scale_part[part][col] = sum;
+  }
+  __syncthreads();
+
+  // one thread per output of the strip: token = t / 16, row = t % 16, so a token's outputs sit in
+  // 16 consecutive lanes
+  const int t = threadIdx.x;
+  if (t >= 256) return;       // (with 4 waves every thread has an output)
+  const int token = t >> 4, nn = t & 15, n = block_row + nn;
+  const int from_lane = (nn >> 2) * 16 + token, from_j = nn & 3;    // where the MFMA left this output
+  float value = 0.f;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) value += partial[w][from_lane][from_j];
+  if (a.ssq_in != nullptr) {
+    float ssq = 0.f;
+#pragma unroll
+    for (int part = 0; part < WAVES * 4; ++part) ssq += scale_part[part][token];
+    value *= rsqrtf(ssq * a.inv_width + a.eps);
+  }
+  const bool live = token < a.M && nn < a.rows_per_block && n < a.N;
+  if (live && a.bias != nullptr) value += bf16_bits_to_float(a.bias[n]);
+
+  if (EPILOGUE == kEpilogueStore) {
+    if (live) a.y[static_cast<size_t>(token) * a.N + n] = value;
+  } else if (EPILOGUE == kEpilogueSilu) {
+    const float up = __shfl_down(value, 1, 64);          // the odd row next to this even one
+    if (live && (nn & 1) == 0) {
+      const float gated = (value / (1.f + expf(-value))) * up;
+      a.act[static_cast<size_t>(token) * (a.N / 2) + (n >> 1)] = __bfloat16_as_ushort(__float2bfloat16(gated));
+    }
+  } else {
+    float updated = 0.f;
+    if (live) {
+      float* place = a.residual + static_cast<size_t>(token) * a.N + n;
+      updated = *place + value;
+      *place = updated;
+      if (a.xg != nullptr) {
+        const float g = a.next_weight != nullptr ? bf16_bits_to_float(a.next_weight[n]) : a.next_weight_f32[n];
+        a.xg[static_cast<size_t>(token) * a.N + n] = __bfloat16_as_ushort(__float2bfloat16(updated * g));
+      }
+    }
+    if (a.ssq_out != nullptr) {
+      float square = updated * updated;
+      square += __shfl_xor(square, 1, 64);
+      square += __shfl_xor(square, 2, 64);
+      square += __shfl_xor(square, 4, 64);
+      square += __shfl_xor(square, 8, 64);
+      if (nn == 0) a.ssq_out[blockIdx.x * 16 + token] = square;      // one row of partial sums per block of W's rows
+    }
+  }
+}
+
+// residual[t, :] = table[token[t], :] as float; and for the first norm, as the residual epilogue
+// above leaves them: xg = bfloat16(residual * g), partial sums of squares per 16 columns.
+template <typename W, typename G>
+__global__ void embed_rows_kernel(const int* __restrict__ tokens, const W* __restrict__ table,
+                                  float* __restrict__ residual, const G* __restrict__ next_weight,
+                                  uint16_t* __restrict__ xg, float* __restrict__ ssq_out, int hidden) {
+  const int t = blockIdx.x;
+  const W* row = table + static_cast<size_t>(tokens[t]) * hidden;
+  for (int base = 0; base < hidden; base += blockDim.x) {
+    const int i = base + threadIdx.x;
+    float value = 0.f;
+    if (i < hidden) {
+      value = to_float(row[i]);
+      residual[static_cast<size_t>(t) * hidden + i] = value;
+      xg[static_cast<size_t>(t) * hidden + i] = __bfloat16_as_ushort(__float2bfloat16(value * to_float(next_weight[i])));
+    }
+    float square = value * value;
+    square += __shfl_xor(square, 1, 64);
+    square += __shfl_xor(square, 2, 64);
+    square += __shfl_xor(square, 4, 64);
+    square += __shfl_xor(square, 8, 64);
+    if ((threadIdx.x & 15) == 0 && i < hidden) ssq_out[(i >> 4) * 16 + t] = square;
+  }
+}
+
+}  // namespace tlie
+
+using namespace tlie;
+
+// x [M, K], w [N, K], bias [N] or null: bfloat16; M <= 16, K % 8 == 0.
+// ssq_in [strips_in, 16] or null (then no row scale); width: the normed input's width.
+// epilogue 0: y float [M, N].  1: act bfloat16 [M, N / 2], N even, W's rows alternating gate, up.
+// 2: residual float [M, N] += y; if xg is given, next_weight [N] (bfloat16 if next_weight_dtype is 1,
+// else float) and xg bfloat16 [M, N]; if ssq_out is given, float [ceil(N / rows_per_block), 16] (all of it is
+// written).
+// waves: 4, 8 or 16, how many waves of a workgroup share K.  rows_per_block: 16 or 8.
+extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, int M, int N, int K, const float* ssq_in,
+                              int strips_in, int width, float eps, int epilogue, float* y, void* act, float* residual,
+                              const void* next_weight, int next_weight_dtype, void* xg, float* ssq_out, int waves,
+                              int rows_per_block, void* stream) {
+  if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K & 7) != 0 || (waves != 4 && waves != 8 && waves != 16)) return kBadArgument;
+  if (rows_per_block != 16 && rows_per_block != 8) return kBadArgument;
+  if (ssq_in != nullptr && (strips_in <= 0 || width <= 0)) return kBadArgument;
+  if (epilogue == kEpilogueStore && y == nullptr) return kBadArgument;
+  if (epilogue == kEpilogueSilu && (act == nullptr || (N & 1) != 0)) return kBadArgument;
+  if (epilogue == kEpilogueResidual && (residual == nullptr || (xg != nullptr && next_weight == nullptr))) return kBadArgument;
+  RowsArgs a;
+  a.x = (const uint16_t*)x, a.w = (const uint16_t*)w, a.bias = (const uint16_t*)bias;
+  a.M = M, a.N = N, a.K = K, a.rows_per_block = rows_per_block;
+  a.k_per_wave = ((K + waves - 1) / waves + 63) / 64 * 64;
+  a.ssq_in = ssq_in, a.strips_in = strips_in, a.inv_width = width > 0 ? 1.f / static_cast<float>(width) : 0.f, a.eps = eps;
+  a.y = y, a.act = (uint16_t*)act, a.residual = residual;
+  a.next_weight = next_weight_dtype == kBF16 ? (const uint16_t*)next_weight : nullptr;
+  a.next_weight_f32 = next_weight_dtype == kBF16 ? nullptr : (const float*)next_weight;
+  a.xg = (uint16_t*)xg, a.ssq_out = ssq_out;
+  const dim3 grid((N + rows_per_block - 1) / rows_per_block);
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(E)                                                                                  \
+  if (epilogue == E) {                                                                                \
+    if (waves == 16)                                                                                  \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 16>), grid, dim3(1024), 0, s, a);                        \
+    else if (waves == 8)                                                                              \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 8>), grid, dim3(512), 0, s, a);                          \
+    else                                                                                              \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 4>), grid, dim3(256), 0, s, a);                          \
+    return launch_status();                                                                           \
+  }
+  TLIE_CASE(kEpilogueStore)
+  TLIE_CASE(kEpilogueSilu)
+  TLIE_CASE(kEpilogueResidual)
+#undef TLIE_CASE
+  return kBadArgument;
+}
+
+// tokens [T] (T <= 16), table [vocab, hidden]; residual float [T, hidden]; next_weight [hidden];
+// xg bfloat16 [T, hidden]; ssq_out float [ceil(hidden / 16), 16].
+extern "C" int tlie_embed_rows(const int* tokens, const void* table, int table_dtype, float* residual,
+                               const void* next_weight, int next_weight_dtype, void* xg, float* ssq_out, int num_tokens,
+                               int hidden, void* stream) {
+  if (num_tokens <= 0 || num_tokens > 16 || hidden <= 0) return kBadArgument;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(num_tokens), block(256);
+#define TLIE_CASE(WC, W, GC, G)                                                                                      \
+  if (table_dtype == WC && next_weight_dtype == GC) {                                                                \
+    hipLaunchKernelGGL((embed_rows_kernel<W, G>), grid, block, 0, s, tokens, (const W*)table, residual,               \
+                       (const G*)next_weight, (uint16_t*)xg, ssq_out, hidden);                                       \
+    return launch_status();                                                                                          \
+  }
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+  TLIE_CASE(kF32, float, kF32, float)
+#undef TLIE_CASE
+  return kBadArgument;
+}

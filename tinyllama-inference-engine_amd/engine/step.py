@@ -54,6 +54,8 @@ class StepContext:
     want_rows: torch.Tensor        # int32 [num_wanted] token indices
     groups: list[GroupView]
     host: dict                     # the same arrays as numpy, by name
+    few_rows: bool = False         # at most 16 tokens of bfloat16: the step may use the products that fold norms and adds in
+    wants_all_rows: bool = False   # the wanted rows are all the step's tokens, in order
     _tiles: dict = field(default_factory=dict)
 
     def attention_tiles(self, groups_per_kv: int, num_kv_heads: int, head_dim: int):
@@ -122,7 +124,7 @@ class ModelRunner:
                 raise out_of_bounds(f"request {entry.request!r} would pass the model's {limit} positions")
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        return build_context(self.cache, entries, self.device)
+        return build_context(self.cache, entries, self.device, few_rows_dtype=self.model.dtype)
 
     # ---- the step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -195,7 +197,8 @@ class DecodeGraph:
             num_tokens=bucket, num_seqs=bucket, num_wanted=bucket, max_new=1, max_context=longest, tokens=views["tokens"],
             positions=views["positions"], token_seq=views["token_seq"], no_slots=views["no_slots"],
             seq_start=views["seq_start"], seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"],
-            seq_slot=views["seq_slot"], want_rows=views["want_rows"], groups=groups, host=self.host)
+            seq_slot=views["seq_slot"], want_rows=views["want_rows"], groups=groups, host=self.host,
+            few_rows=bucket <= 16 and runner.model.dtype == torch.bfloat16, wants_all_rows=True)
         self.graph = None
         self.logits = None
 
@@ -237,7 +240,7 @@ class DecodeGraph:
         return self.logits[:len(entries)]
 
 
-def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> StepContext:
+def build_context(cache: CacheManager, entries: Sequence[StepEntry], device, few_rows_dtype=None) -> StepContext:
     """The step's arrays for entries whose pages are reserved: built on the host, sent in one
     transfer."""
     counts = [len(entry.tokens) for entry in entries]
@@ -286,5 +289,7 @@ def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> 
         max_context=int(host["seq_len"].max()), tokens=views["tokens"], positions=views["positions"],
         token_seq=views["token_seq"], no_slots=views["no_slots"], seq_start=views["seq_start"],
         seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
-        want_rows=views["want_rows"], groups=groups, host=host)
+        want_rows=views["want_rows"], groups=groups, host=host,
+        few_rows=total <= 16 and few_rows_dtype == torch.bfloat16,
+        wants_all_rows=bool(want_rows.size == total and np.array_equal(want_rows, np.arange(total))))
 

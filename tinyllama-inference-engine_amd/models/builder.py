@@ -7,6 +7,7 @@ import torch
 from .. import parts as _parts  # noqa: F401  (fills the part registries)
 from ..cache.manager import RunNeed
 from ..config.spec import ModelSpec, TensorSpec
+from ..ops import ResidualUpdated
 from ..registry import lookup
 
 
@@ -60,13 +61,22 @@ class DecoderModel:
 
     def forward(self, ctx, bindings) -> torch.Tensor:
         """Runs the step's tokens; returns float32 logits [wanted rows, vocab]."""
-        residual = self.embedding.forward(ctx.tokens)
-        pending = None
-        for index, run in enumerate(self.spec.runs):
-            pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index])
+        runs = self.spec.runs
+        first_norm = self.blocks[runs[0].layer].mixer_norm
+        if ctx.few_rows and hasattr(self.embedding, "forward_rows") and first_norm.lazy_params() is not None:
+            residual, normed = self.embedding.forward_rows(ctx.tokens, first_norm.lazy_params())
+            pending = ResidualUpdated(normed)
+        else:
+            residual, pending = self.embedding.forward(ctx.tokens), None
+        for index, run in enumerate(runs):
+            next_norm = self.blocks[runs[index + 1].layer].mixer_norm if index + 1 < len(runs) else self.final_norm
+            pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index], next_norm=next_norm)
         if ctx.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
-        normed = self.final_norm.add_forward(residual, pending, rows=ctx.want_rows)
+        if ctx.wants_all_rows:
+            normed = self.final_norm.add_forward(residual, pending, lazy=ctx.few_rows and self.head.takes_normed_rows(residual.shape[0]))
+        else:
+            normed = self.final_norm.add_forward(residual, pending, rows=ctx.want_rows)
         return self.head.forward(normed)
 
 

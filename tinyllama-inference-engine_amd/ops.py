@@ -143,8 +143,9 @@ def add_rmsnorm(residual: torch.Tensor, delta: Product | None, weight: torch.Ten
     return out
 
 
-def silu_mul(gate_up: Product, out_dtype: torch.dtype) -> torch.Tensor:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, inter + i]."""
+def silu_mul(gate_up: Product, out_dtype: torch.dtype, interleaved: bool = False) -> torch.Tensor:
+    """out[t, i] = silu(gate[t, i]) * up[t, i], with gate_up = [gate | up] side by side or, interleaved,
+    g0 u0 g1 u1 ..."""
     _check_product(gate_up, "gate_up")
     if gate_up.cols % 2 != 0:
         raise invalid_shape("silu_mul: the input holds gate and up side by side, its width must be even")
@@ -152,7 +153,7 @@ def silu_mul(gate_up: Product, out_dtype: torch.dtype) -> torch.Tensor:
     out = torch.empty((rows, inter), dtype=out_dtype, device=gate_up.data.device)
     _check(library().tlie_silu_mul(_ptr(gate_up.data), dtype_code(gate_up.data.dtype), gate_up.nsplit,
                                    ctypes.c_longlong(gate_up.split_stride), _ptr(out), dtype_code(out_dtype), rows, inter,
-                                   _stream()), "silu_mul")
+                                   1 if interleaved else 0, _stream()), "silu_mul")
     return out
 
 
@@ -387,3 +388,132 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
                                          split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
                                          int(window) if window else 0, ctypes.c_float(scale), _stream()), "attention_mfma")
     return out
+
+
+# ---- at most 16 rows: products with the layer's neighbouring arithmetic folded in --------------------
+ROWS_MAX = 16
+
+
+@dataclass
+class NormedRows:
+    """The input of a product, not yet normed: xg = bfloat16(residual * norm weight) [T, width] and
+    partial sums of squares of the residual's rows, ssq [parts, 16] (each part covers some of the
+    columns; their sum over the parts is the row's sum of squares).  The product applies
+    rsqrt(sum(ssq) / width + eps) to its result's rows, which is the same as having normed the
+    input."""
+    xg: torch.Tensor
+    ssq: torch.Tensor
+    eps: float
+
+    @property
+    def shape(self):
+        return self.xg.shape
+
+
+@dataclass
+class ResidualUpdated:
+    """A product's result was added into the residual by the kernel that computed it; `normed`
+    is the residual as the next norm's product wants it, when that was asked for."""
+    normed: NormedRows | None
+
+
+def gemm_rows_takes(rows: int, weight: torch.Tensor, dtype: torch.dtype) -> bool:
+    return (dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < rows <= ROWS_MAX
+            and weight.shape[1] % 8 == 0)
+
+
+def gemm_rows_shape(out_features: int, in_features: int) -> tuple[int, int]:
+    """(waves that share K, rows of W per workgroup).  A workgroup per 16 rows; per 8 when that
+    would leave CUs without one (the chip has 256).  Measured on the TinyLlama shapes: 4 waves
+    when the strips alone fill the chip several times over, 16 for a long K, else 8."""
+    rows_per_block = 16 if (out_features + 15) // 16 >= 256 else 8
+    blocks = (out_features + rows_per_block - 1) // rows_per_block
+    waves = 16 if in_features > 4096 else (4 if blocks >= 2048 else 8)
+    return waves, rows_per_block
+
+
+def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str = "store",
+              residual: torch.Tensor | None = None, next_norm: tuple | None = None, waves: int | None = None,
+              rows_per_block: int | None = None):
+    """y = x . W^T (+ bias) for at most 16 rows.  x: bfloat16 [M, K], or `NormedRows` (then the
+    result's rows are scaled as the norm would have scaled the input).
+    epilogue "store": float32 [M, N] as a `Product`.  "silu": W's rows alternate gate and up;
+    returns bfloat16 silu(gate) * up [M, N / 2].  "residual": residual [M, N] += y in place, returns
+    a `ResidualUpdated`, with the next norm's inputs when next_norm = (weight [N], eps) is given."""
+    scale = x if isinstance(x, NormedRows) else None
+    data = scale.xg if scale is not None else x
+    _device_tensor(data, "x", torch.bfloat16)
+    _device_tensor(weight, "weight", torch.bfloat16)
+    if data.dim() != 2 or weight.dim() != 2 or data.shape[1] != weight.shape[1]:
+        raise invalid_shape(f"gemm_rows: x {list(data.shape)} and weight {list(weight.shape)} do not fit")
+    rows, (out_features, in_features) = data.shape[0], weight.shape
+    if not gemm_rows_takes(rows, weight, data.dtype):
+        raise invalid_argument(f"gemm_rows takes 1..{ROWS_MAX} rows of bfloat16 and an inner size that is a multiple of 8")
+    if bias is not None:
+        _device_tensor(bias, "bias", torch.bfloat16)
+        if bias.shape != (out_features,):
+            raise invalid_shape("gemm_rows: bias needs one entry per output")
+    ssq_in, strips_in, eps = None, 0, 0.0
+    if scale is not None:
+        _device_tensor(scale.ssq, "ssq", torch.float32)
+        if scale.ssq.dim() != 2 or scale.ssq.shape[1] != 16 or scale.ssq.shape[0] == 0:
+            raise invalid_shape(f"gemm_rows: ssq {list(scale.ssq.shape)} is not [parts, 16]")
+        ssq_in, strips_in, eps = scale.ssq, scale.ssq.shape[0], float(scale.eps)
+    default_waves, default_rows = gemm_rows_shape(out_features, in_features)
+    waves, rows_per_block = waves or default_waves, rows_per_block or default_rows
+    if epilogue == "silu" and rows_per_block % 2 != 0:
+        raise invalid_argument("gemm_rows: a gate and its up must fall into one block")
+    device = data.device
+    y = act = xg = ssq_out = next_weight = None
+    next_code = BF16
+    if epilogue == "store":
+        code = 0
+        y = torch.empty((rows, out_features), dtype=torch.float32, device=device)
+    elif epilogue == "silu":
+        code = 1
+        if out_features % 2 != 0:
+            raise invalid_shape("gemm_rows: the gated product needs an even number of rows of W")
+        act = torch.empty((rows, out_features // 2), dtype=torch.bfloat16, device=device)
+    elif epilogue == "residual":
+        code = 2
+        _device_tensor(residual, "residual", torch.float32)
+        if residual.shape != (rows, out_features):
+            raise invalid_shape(f"gemm_rows: residual {list(residual.shape)} is not [{rows}, {out_features}]")
+        if next_norm is not None:
+            next_weight = next_norm[0]
+            _device_tensor(next_weight, "next norm weight", (torch.bfloat16, torch.float32))
+            if next_weight.shape != (out_features,):
+                raise invalid_shape("gemm_rows: the next norm's weight needs one entry per output")
+            next_code = dtype_code(next_weight.dtype)
+            xg = torch.empty((rows, out_features), dtype=torch.bfloat16, device=device)
+            ssq_out = torch.empty(((out_features + rows_per_block - 1) // rows_per_block, 16), dtype=torch.float32, device=device)
+    else:
+        raise invalid_argument(f"gemm_rows: unknown epilogue '{epilogue}'")
+    _check(library().tlie_gemm_rows(_ptr(data), _ptr(weight), _ptr(bias), rows, out_features, in_features, _ptr(ssq_in),
+                                    strips_in, in_features, ctypes.c_float(eps), code, _ptr(y), _ptr(act), _ptr(residual),
+                                    _ptr(next_weight), next_code, _ptr(xg), _ptr(ssq_out), waves, rows_per_block, _stream()),
+           "gemm_rows")
+    if epilogue == "store":
+        return Product(y, 1)
+    if epilogue == "silu":
+        return act
+    return ResidualUpdated(NormedRows(xg, ssq_out, float(next_norm[1])) if next_norm is not None else None)
+
+
+def embed_rows(tokens: torch.Tensor, table: torch.Tensor, next_norm: tuple):
+    """The embedding for at most 16 tokens with the first norm's inputs: returns (float32
+    residual [T, hidden], NormedRows)."""
+    _device_tensor(tokens, "tokens", torch.int32)
+    _device_tensor(table, "embedding table", (torch.float32, torch.bfloat16))
+    next_weight, next_eps = next_norm
+    _device_tensor(next_weight, "next norm weight", (torch.bfloat16, torch.float32))
+    if tokens.dim() != 1 or table.dim() != 2 or next_weight.shape != (table.shape[1],) or not 0 < tokens.shape[0] <= ROWS_MAX:
+        raise invalid_shape("embed_rows takes 1..16 tokens, a table [vocab, hidden] and a norm weight [hidden]")
+    count, hidden = tokens.shape[0], table.shape[1]
+    residual = torch.empty((count, hidden), dtype=torch.float32, device=table.device)
+    xg = torch.empty((count, hidden), dtype=torch.bfloat16, device=table.device)
+    ssq = torch.empty(((hidden + 15) // 16, 16), dtype=torch.float32, device=table.device)
+    _check(library().tlie_embed_rows(_ptr(tokens), _ptr(table), dtype_code(table.dtype), _ptr(residual), _ptr(next_weight),
+                                     dtype_code(next_weight.dtype), _ptr(xg), _ptr(ssq), count, hidden, _stream()),
+           "embed_rows")
+    return residual, NormedRows(xg, ssq, float(next_eps))

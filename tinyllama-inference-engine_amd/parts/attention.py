@@ -66,10 +66,15 @@ class Attention(Mixer):
         # a position encoding applied as tensors may do anything; a rotation table (or none) is fused
         return self.position.rotary_table() is not None or type(self.position).apply_qk is PositionEncoding.apply_qk
 
+    adds_to_residual = True
+
+    def takes_normed_rows(self, rows: int) -> bool:
+        return self.qkv.takes_rows(rows)
+
     def cache_need(self):
         return KVCacheNeed(self.nkv, self.d, int(self.window) if self.window is not None else None)
 
-    def forward(self, x, ctx, binding: Binding):
+    def forward(self, x, ctx, binding: Binding, into=None):
         pages = ctx.groups[binding.group]
         qkv = self.qkv(x)
         slot_map = pages.slot_map if binding.writes else ctx.no_slots
@@ -87,7 +92,7 @@ class Attention(Mixer):
         else:
             attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
                                              self.nkv, self.d, self.window, self.scale)
-        return self.o(attended)
+        return self.o(attended, into=into)
 
     def _apply_other_positions(self, qkv, ctx):
         """A position encoding that is no rotation table: applied to q and k as tensors."""

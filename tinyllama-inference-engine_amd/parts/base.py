@@ -11,6 +11,7 @@ what the cache manager holds for it arrives in the `Binding`.
     Mixer          forward(x [T, H], ctx, binding) -> Product or tensor [T, H]
                    cache_need() -> KVCacheNeed | None;  state_need() -> StateNeed | None
     FeedForward    forward(x [T, H], ctx) -> Product or tensor [T, H]
+                   (both may opt into the fusions of steps of few rows, see Mixer below)
     PositionEncoding
                    rotary_table() -> (inv_freq, rot_dim) | None   (lets attention fuse it)
                    apply_qk(q, k, positions) -> (q, k)             (any other scheme)
@@ -24,7 +25,7 @@ from typing import Any
 import torch
 
 from ..config.spec import PartSpec, TensorSpec
-from ..ops import Product, as_product
+from ..ops import NormedRows, Product, ResidualUpdated, as_product
 
 
 @dataclass(frozen=True)
@@ -71,12 +72,30 @@ class Part:
         pass
 
 
+@dataclass
+class ResidualTarget:
+    """Handed to a mixer or feed-forward that can add its result into the residual itself (in the
+    kernel of its last product): the float32 residual, and (weight, eps) of the norm that reads the
+    residual next, or None."""
+    residual: torch.Tensor
+    next_norm: tuple | None = None
+
+
 class Norm(Part):
     def forward(self, residual: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
-    def add_forward(self, residual: torch.Tensor, delta, rows: torch.Tensor | None = None) -> torch.Tensor:
-        """Unfused default: add in place, then norm; with `rows`, norm those rows of the sum only."""
+    def lazy_params(self):
+        """(weight, eps) when this norm can be folded into the product that follows it (its
+        weight applied to the residual by whoever writes the residual, its scale to the product's
+        rows), else None."""
+        return None
+
+    def add_forward(self, residual: torch.Tensor, delta, rows: torch.Tensor | None = None, lazy: bool = False):
+        """Unfused default: add in place, then norm; with `rows`, norm those rows of the sum only.
+        `delta` may be a `ResidualUpdated`: then the residual already holds it."""
+        if isinstance(delta, ResidualUpdated):
+            delta = None
         if rows is not None:
             picked = residual[rows.long()]
             if delta is not None:
@@ -105,11 +124,27 @@ class Mixer(Part):
     def forward(self, x: torch.Tensor, ctx: Any, binding: Binding):
         raise NotImplementedError
 
+    # A mixer (or feed-forward) may offer two things to a block that runs a step of few rows:
+    #   takes_normed_rows(rows) -> True: `x` may be a `NormedRows` (the norm before it is folded
+    #       into its first product);
+    #   adds_to_residual = True: `forward(..., into=ResidualTarget)` adds the result into the
+    #       residual itself and returns a `ResidualUpdated` (or, when it cannot for this step, its
+    #       result as usual).
+    adds_to_residual = False
+
+    def takes_normed_rows(self, rows: int) -> bool:
+        return False
+
 
 class FeedForward(Part):
+    adds_to_residual = False
+
+    def takes_normed_rows(self, rows: int) -> bool:
+        return False
+
     def forward(self, x: torch.Tensor, ctx: Any):
         raise NotImplementedError
 
 
 __all__ = ["KVCacheNeed", "StateNeed", "Binding", "Part", "Norm", "PositionEncoding", "Mixer", "FeedForward",
-           "Product", "as_product"]
+           "Product", "as_product", "NormedRows", "ResidualUpdated", "ResidualTarget"]

@@ -10,6 +10,7 @@ from __future__ import annotations
 
 from ..config.spec import LayerSpec
 from ..registry import lookup, register
+from .base import ResidualTarget
 
 
 @register("block", "pre_norm")
@@ -44,8 +45,20 @@ class PreNormBlock:
         return all(getattr(part, "graph_safe", False)
                    for part in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward))
 
-    def forward(self, residual, pending, ctx, binding):
-        normed = self.mixer_norm.add_forward(residual, pending)
-        mixed = self.mixer.forward(normed, ctx, binding)
-        normed = self.feed_forward_norm.add_forward(residual, mixed)
+    def forward(self, residual, pending, ctx, binding, next_norm=None):
+        """`pending`: what the residual still lacks (a product, a `ResidualUpdated`, or None).
+        `next_norm`: the norm that reads the residual after this block, if the caller knows it.
+        In a step of few rows the parts that offer it fold the norms into their products and add
+        their results into the residual themselves; otherwise the norm kernels do both."""
+        rows = residual.shape[0]
+        few = ctx.few_rows
+        normed = self.mixer_norm.add_forward(residual, pending, lazy=few and self.mixer.takes_normed_rows(rows))
+        if few and self.mixer.adds_to_residual:
+            mixed = self.mixer.forward(normed, ctx, binding, into=ResidualTarget(residual, self.feed_forward_norm.lazy_params()))
+        else:
+            mixed = self.mixer.forward(normed, ctx, binding)
+        normed = self.feed_forward_norm.add_forward(residual, mixed, lazy=few and self.feed_forward.takes_normed_rows(rows))
+        if few and self.feed_forward.adds_to_residual:
+            return self.feed_forward.forward(normed, ctx, into=ResidualTarget(
+                residual, next_norm.lazy_params() if next_norm is not None else None))
         return self.feed_forward.forward(normed, ctx)

@@ -34,6 +34,10 @@ class TokenEmbedding(Part):
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
         return ops.embed_gather(tokens, self.table)
 
+    def forward_rows(self, tokens: torch.Tensor, next_norm: tuple):
+        """For a step of few rows: the residual and the first norm's inputs in one launch."""
+        return ops.embed_rows(tokens, self.table, next_norm)
+
 
 @register("head", "lm_head")
 class LMHead(Part):
@@ -55,5 +59,8 @@ class LMHead(Part):
         matrix = weights[TokenEmbedding.NAME] if self.tied else weights[self.NAME]
         self.linear = Linear(matrix, None, self.dtype)
 
-    def forward(self, normed: torch.Tensor) -> torch.Tensor:
+    def takes_normed_rows(self, rows: int) -> bool:
+        return self.linear.takes_rows(rows)
+
+    def forward(self, normed) -> torch.Tensor:
         return self.linear(normed, out_dtype=torch.float32, whole=True).dense(torch.float32)

@@ -4,6 +4,8 @@
 Which kernel runs is decided here and nowhere else:
   float32 activations            the true 32-bit kernel (plain FMAs, no matrix instruction)
   bfloat16, weight kept float32  the same kernel on widened values
+  bfloat16, at most 16 rows      the rows kernel when the caller folds something in: the norm before the
+                                 product, the SiLU gate or the add into the residual after it
   bfloat16, at most 64 rows      the skinny MFMA kernel (W streamed once, split-K partial sums)
   bfloat16, more rows            the library's product (as the reference uses a library for its
                                  products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out
@@ -26,11 +28,29 @@ class Linear:
         self.dtype = dtype
         self.out_features, self.in_features = self.weight.shape
 
-    def __call__(self, x: torch.Tensor, out_dtype: torch.dtype | None = None, whole: bool = False) -> Product:
+    def takes_rows(self, rows: int) -> bool:
+        """Whether a step of `rows` rows can go to the rows kernel (and so may bring a `NormedRows`,
+        ask for the gate, or for the add into the residual)."""
+        return ops.gemm_rows_takes(rows, self.weight, self.dtype)
+
+    def __call__(self, x, out_dtype: torch.dtype | None = None, whole: bool = False, into=None, gated: bool = False):
         """out_dtype: what a dense result is stored in (the skinny kernel's partial sums are float32
         whatever it says).  whole: the caller has no kernel that adds partial sums up, so the
-        product must come as one array (the skinny kernel then does not split K)."""
+        product must come as one array (the skinny kernel then does not split K).
+        into (a `ResidualTarget`): add the result into the residual, if the kernel for this step can
+        (then a `ResidualUpdated` comes back, else the result as usual).  gated: the weight's rows
+        alternate gate and up; if the kernel for this step can, silu(gate) * up comes back as a
+        tensor, else the product as usual."""
         out_dtype = out_dtype or self.dtype
+        if self.takes_rows(x.shape[0]):
+            if into is not None:
+                return ops.gemm_rows(x, self.weight, self.bias, "residual", residual=into.residual, next_norm=into.next_norm)
+            if gated:
+                return ops.gemm_rows(x, self.weight, self.bias, "silu")
+            if isinstance(x, ops.NormedRows):
+                return ops.gemm_rows(x, self.weight, self.bias, "store")
+        if isinstance(x, ops.NormedRows):
+            raise ops.invalid_argument("this product cannot fold the norm before it; ask takes_rows() first")
         if ops.gemm_skinny_takes(x, self.weight) and (not whole or out_dtype == torch.float32):
             split_len = (self.in_features + 63) // 64 * 64 if whole else None
             return ops.gemm_skinny(x, self.weight, self.bias, split_len=split_len)

@@ -1,6 +1,7 @@
 """The SiLU-gated feed-forward: down(silu(gate(x)) * up(x)) (src/model.cpp:187-196 of the
 reference; SiluMultiply, src/operators.cpp:157-159).  gate and up are one product over the
-concatenated weight [2 * inter, hidden]."""
+weight [2 * inter, hidden] whose rows alternate gate and up (g0, u0, g1, u1, ...): the product of
+few rows then has a gate and its up in one lane and applies the activation itself."""
 from __future__ import annotations
 
 import torch
@@ -35,9 +36,17 @@ class GatedMLP(FeedForward):
                 TensorSpec(prefix + "down_proj.weight", (hidden, inter))]
 
     def load(self, weights, prefix):
-        self.gate_up = Linear(torch.cat([weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]], dim=0),
-                              None, self.dtype)
+        gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
+        self.gate_up = Linear(torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden), None, self.dtype)
         self.down = Linear(weights[prefix + "down_proj.weight"], None, self.dtype)
 
-    def forward(self, x, ctx):
-        return self.down(ops.silu_mul(self.gate_up(x), self.dtype))
+    adds_to_residual = True
+
+    def takes_normed_rows(self, rows: int) -> bool:
+        return self.gate_up.takes_rows(rows)
+
+    def forward(self, x, ctx, into=None):
+        hidden = self.gate_up(x, gated=True)
+        if isinstance(hidden, ops.Product):
+            hidden = ops.silu_mul(hidden, self.dtype, interleaved=True)
+        return self.down(hidden, into=into)

@@ -8,7 +8,7 @@ import torch
 from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..registry import register
-from .base import Norm, as_product
+from .base import Norm, ResidualUpdated, as_product
 
 
 @register("norm", "rms_norm")
@@ -32,6 +32,15 @@ class RMSNorm(Norm):
     def forward(self, residual):
         return ops.add_rmsnorm(residual, None, self.weight, self.eps, self.dtype)
 
-    def add_forward(self, residual, delta, rows=None):
+    def lazy_params(self):
+        return self.weight, self.eps
+
+    def add_forward(self, residual, delta, rows=None, lazy=False):
+        if isinstance(delta, ResidualUpdated):
+            # the residual holds the sum already; if its writer also left this norm's inputs and the
+            # reader can fold the norm into its product, nothing is launched here
+            if lazy and rows is None and delta.normed is not None:
+                return delta.normed
+            delta = None
         product = as_product(delta) if delta is not None else None
         return ops.add_rmsnorm(residual, product, self.weight, self.eps, self.dtype, rows=rows)
