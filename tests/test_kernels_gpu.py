@@ -517,3 +517,46 @@ def test_embed_rows_and_refusals():
     with pytest.raises(EngineError):
         ops.gemm_rows(torch.randn(2, 64, device=DEV).bfloat16(), torch.randn(7, 64, device=DEV).bfloat16(), None, "silu")
     assert not ops.gemm_rows_takes(4, torch.randn(8, 12, device=DEV).bfloat16(), torch.bfloat16)
+
+
+@pytest.mark.parametrize("case", [dict(nq=5, nkv=3, d=48, rot=48, page=8), dict(nq=4, nkv=1, d=64, rot=32, page=16),
+                                  dict(nq=2, nkv=2, d=16, rot=0, page=16), dict(nq=32, nkv=4, d=64, rot=64, page=16)])
+def test_rotation_in_paired_order_and_inside_the_product(case):
+    """The fused q/k/v weight's rows may be stored with rotation pairs side by side.  The rotation
+    kernel reading such columns, and the product of few rows that rotates and writes the cache
+    itself, must give what the plain order through the plain kernels gives."""
+    from tlie_amd import ops
+    nq, nkv, d, rot, page = case["nq"], case["nkv"], case["d"], case["rot"], case["page"]
+    tokens, hidden = 7, 72
+    torch.manual_seed(d + rot)
+    x = torch.randn(tokens, hidden).bfloat16().to(DEV)
+    w = (torch.randn((nq + 2 * nkv) * d, hidden) / math.sqrt(hidden)).bfloat16().to(DEV)
+    b = torch.randn((nq + 2 * nkv) * d).bfloat16().to(DEV)
+    positions = torch.tensor([0, 1, 77, 4095, 5, 6, 300], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([3, 12, -1, 40, 41, 7, 0], dtype=torch.int32, device=DEV)
+    inv_freq = None
+    if rot:
+        inv_freq = torch.pow(torch.tensor(10000.0), -2.0 * torch.arange(rot // 2, dtype=torch.float32) / rot).to(DEV)
+
+    def fresh_cache():
+        return torch.full((8, 2, nkv, page * d), -3.0, dtype=torch.bfloat16, device=DEV)
+    plain_cache = fresh_cache()
+    plain_q = ops.rope_cache(ops.gemm_skinny(x, w, b), positions, slots, inv_freq, rot, plain_cache, nq, nkv, d, torch.bfloat16)
+    order = ops.paired_rows(nq, nkv, d, rot).to(DEV)
+    assert sorted(order.tolist()) == list(range((nq + 2 * nkv) * d))
+    if rot:
+        assert order[:4].tolist() == [0, rot // 2, 1, rot // 2 + 1]
+    w_paired, b_paired = w[order].contiguous(), b[order].contiguous()
+    paired_cache = fresh_cache()
+    paired_q = ops.rope_cache(ops.gemm_skinny(x, w_paired, b_paired), positions, slots, inv_freq, rot, paired_cache, nq, nkv, d,
+                              torch.bfloat16, paired=True)
+    assert torch.equal(paired_q, plain_q) and torch.equal(paired_cache, plain_cache)
+    for rows_per_block in (8, 16):
+        fused_cache = fresh_cache()
+        target = ops.RopeTarget(positions, slots, inv_freq, rot, fused_cache, nq, nkv, d)
+        fused_q = ops.gemm_rows(x, w_paired, b_paired, "rope", rope=target, rows_per_block=rows_per_block)
+        # the two products sum in another order, so the last bit of a bfloat16 may differ
+        assert rel_err(fused_q, plain_q.double()) < 1e-2
+        assert rel_err(fused_cache, plain_cache.double()) < 1e-2
+        untouched = plain_cache == -3.0
+        assert torch.equal(fused_cache[untouched], plain_cache[untouched])

@@ -26,6 +26,11 @@
 //   * residual: residual[m, n] += y (float32, in place: every element has one owner), and for the
 //     norm that reads the residual next: xg[m, n] = bfloat16(residual * g_next[n]) and the partial
 //     sums of squares per row and 16 columns.
+//   * rotation and cache write, for the fused q/k/v projection: the rows of W are stored so that
+//     the two elements of a rotation pair, (i, i + rot_dim / 2) of a head, are neighbours
+//     (positions 2i and 2i + 1); a pair then sits in two adjacent lanes, is turned by the token's
+//     angle, and goes to q or to the cache row of the token's slot (what rope_cache.hip does as a
+//     kernel of its own for longer steps).
 #include "common.h"
 
 namespace tlie {
@@ -38,7 +43,7 @@ union RowPack {
   bf16x8 v;
 };
 
-constexpr int kEpilogueStore = 0, kEpilogueSilu = 1, kEpilogueResidual = 2;
+constexpr int kEpilogueStore = 0, kEpilogueSilu = 1, kEpilogueResidual = 2, kEpilogueRope = 3;
 
 struct RowsArgs {
   const uint16_t* x;          // [M, K] bfloat16
@@ -58,6 +63,13 @@ struct RowsArgs {
   const float* next_weight_f32; // the same when that weight is kept in float32
   uint16_t* xg;               // residual: [M, N] bfloat16(residual * next weight), or null
   float* ssq_out;             // residual: [ceil(N / rows_per_block), 16], or null
+  // rotation and cache write: N = (nq + 2 nkv) * d, heads in the order q | k | v
+  const int* positions;       // [M]
+  const int* slot_map;        // [M] cache row of each token (page * page_size + row), or -1
+  const float* inv_freq;      // [rot_dim / 2], or null: no rotation
+  int rot_dim, nq, nkv, d, page_size;
+  uint16_t* q_out;            // [M, nq * d]
+  uint16_t* cache;            // [pages, 2, nkv, page_size * d]: keys [row][dim], values [dim][row]
 };
 
 // WAVES: 4, 8 or 16 waves share K (more waves for a long K or few strips, fewer when the strips
@@ -145,6 +157,40 @@ gemm_rows_kernel(const RowsArgs a) {
       const float gated = (value / (1.f + expf(-value))) * up;
       a.act[static_cast<size_t>(token) * (a.N / 2) + (n >> 1)] = __bfloat16_as_ushort(__float2bfloat16(gated));
     }
+  } else if (EPILOGUE == kEpilogueRope) {
+    const float other = __shfl_xor(value, 1, 64);        // the pair's other element, when this one is rotated
+    if (live) {
+      const int head = n / a.d, p = n % a.d;
+      float result = value;
+      int e = p;
+      if (a.inv_freq != nullptr && head < a.nq + a.nkv && p < a.rot_dim) {
+        const int i = p >> 1, half = a.rot_dim >> 1;
+        float sine, cosine;
+        sincosf(static_cast<float>(a.positions[token]) * a.inv_freq[i], &sine, &cosine);
+        if (p & 1) {
+          e = i + half;
+          result = value * cosine + other * sine;        // second' = second cos + first sin
+        } else {
+          e = i;
+          result = value * cosine - other * sine;        // first' = first cos - second sin
+        }
+      }
+      const uint16_t bits = __bfloat16_as_ushort(__float2bfloat16(result));
+      if (head < a.nq) {
+        a.q_out[(static_cast<size_t>(token) * a.nq + head) * a.d + e] = bits;
+      } else {
+        const int slot = a.slot_map[token];
+        if (slot >= 0) {
+          const size_t head_stride = static_cast<size_t>(a.page_size) * a.d;
+          uint16_t* page = a.cache + static_cast<size_t>(slot / a.page_size) * 2 * a.nkv * head_stride;
+          const int row = slot % a.page_size;
+          if (head < a.nq + a.nkv)
+            page[(head - a.nq) * head_stride + static_cast<size_t>(row) * a.d + e] = bits;
+          else
+            page[(head - a.nq) * head_stride + static_cast<size_t>(e) * a.page_size + row] = bits;
+        }
+      }
+    }
   } else {
     float updated = 0.f;
     if (live) {
@@ -203,16 +249,25 @@ using namespace tlie;
 // else float) and xg bfloat16 [M, N]; if ssq_out is given, float [ceil(N / rows_per_block), 16] (all of it is
 // written).
 // waves: 4, 8 or 16, how many waves of a workgroup share K.  rows_per_block: 16 or 8.
+// 3: the rotation and cache write of rope_cache.hip on W's rows in paired order (see above): positions, slot_map [M],
+// inv_freq [rot_dim / 2] or null, q_out bfloat16 [M, nq * d], cache bfloat16 [pages, 2, nkv, page_size * d];
+// N = (nq + 2 nkv) * d.
 extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, int M, int N, int K, const float* ssq_in,
                               int strips_in, int width, float eps, int epilogue, float* y, void* act, float* residual,
-                              const void* next_weight, int next_weight_dtype, void* xg, float* ssq_out, int waves,
-                              int rows_per_block, void* stream) {
+                              const void* next_weight, int next_weight_dtype, void* xg, float* ssq_out,
+                              const int* positions, const int* slot_map, const float* inv_freq, int rot_dim, int nq,
+                              int nkv, int d, int page_size, void* q_out, void* cache, int waves, int rows_per_block,
+                              void* stream) {
   if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K & 7) != 0 || (waves != 4 && waves != 8 && waves != 16)) return kBadArgument;
   if (rows_per_block != 16 && rows_per_block != 8) return kBadArgument;
   if (ssq_in != nullptr && (strips_in <= 0 || width <= 0)) return kBadArgument;
   if (epilogue == kEpilogueStore && y == nullptr) return kBadArgument;
   if (epilogue == kEpilogueSilu && (act == nullptr || (N & 1) != 0)) return kBadArgument;
   if (epilogue == kEpilogueResidual && (residual == nullptr || (xg != nullptr && next_weight == nullptr))) return kBadArgument;
+  if (epilogue == kEpilogueRope &&
+      (positions == nullptr || slot_map == nullptr || q_out == nullptr || cache == nullptr || nq <= 0 || nkv <= 0 || d <= 0 ||
+       page_size <= 0 || N != (nq + 2 * nkv) * d || rot_dim < 0 || rot_dim > d || (rot_dim & 1) != 0 || (d & 1) != 0))
+    return kBadArgument;
   RowsArgs a;
   a.x = (const uint16_t*)x, a.w = (const uint16_t*)w, a.bias = (const uint16_t*)bias;
   a.M = M, a.N = N, a.K = K, a.rows_per_block = rows_per_block;
@@ -222,6 +277,8 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
   a.next_weight = next_weight_dtype == kBF16 ? (const uint16_t*)next_weight : nullptr;
   a.next_weight_f32 = next_weight_dtype == kBF16 ? nullptr : (const float*)next_weight;
   a.xg = (uint16_t*)xg, a.ssq_out = ssq_out;
+  a.positions = positions, a.slot_map = slot_map, a.inv_freq = inv_freq, a.rot_dim = rot_dim;
+  a.nq = nq, a.nkv = nkv, a.d = d, a.page_size = page_size, a.q_out = (uint16_t*)q_out, a.cache = (uint16_t*)cache;
   const dim3 grid((N + rows_per_block - 1) / rows_per_block);
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(E)                                                                                  \
@@ -237,6 +294,7 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
   TLIE_CASE(kEpilogueStore)
   TLIE_CASE(kEpilogueSilu)
   TLIE_CASE(kEpilogueResidual)
+  TLIE_CASE(kEpilogueRope)
 #undef TLIE_CASE
   return kBadArgument;
 }

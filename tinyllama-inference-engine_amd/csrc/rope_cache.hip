@@ -18,12 +18,15 @@ namespace tlie {
 // values at index 1 transposed, [dim][row] (the attention kernels read 4 consecutive rows of one dim).
 // slot_map[t] = page * page_size + row of token t, or -1: nothing is written for that token.
 // rot_dim <= d, even: dimensions from rot_dim on are copied unrotated.  inv_freq may be null
-// (no rotation at all).  blockDim.x = heads_per_block * d; grid = (tokens, ceil(heads / heads_per_block)).
+// (no rotation at all).  paired: within a q or k head the input's columns are stored with the two
+// elements of a rotation pair side by side (element i at 2i, element i + rot_dim/2 at 2i + 1), as
+// the product of few rows wants its weight's rows; outputs are in natural order either way.
+// blockDim.x = heads_per_block * d; grid = (tokens, ceil(heads / heads_per_block)).
 template <typename D, typename A>
 __global__ void rope_cache_kernel(const D* __restrict__ qkv, int nsplit, size_t split_stride,
                                   const int* __restrict__ positions, const int* __restrict__ slot_map,
                                   const float* __restrict__ inv_freq, int rot_dim, A* __restrict__ q_out,
-                                  A* __restrict__ cache, int nq, int nkv, int d, int page_size) {
+                                  A* __restrict__ cache, int nq, int nkv, int d, int page_size, int paired) {
   extern __shared__ float lds[];
   float* cosines = lds;                  // rot_dim / 2
   float* sines = cosines + rot_dim / 2;  // rot_dim / 2
@@ -40,7 +43,9 @@ __global__ void rope_cache_kernel(const D* __restrict__ qkv, int nsplit, size_t 
   const int head = blockIdx.y * (blockDim.x / d) + local_head;
   const bool live = head < heads;
   float mine = 0.f;
-  if (live) mine = sum_splits(qkv + static_cast<size_t>(t) * width + head * d + e, nsplit, split_stride);
+  int column = e;
+  if (paired && head < nq + nkv && e < rot_dim) column = e < half ? 2 * e : 2 * (e - half) + 1;
+  if (live) mine = sum_splits(qkv + static_cast<size_t>(t) * width + head * d + column, nsplit, split_stride);
   values[threadIdx.x] = mine;
   __syncthreads();
   if (!live) return;
@@ -76,7 +81,7 @@ using namespace tlie;
 extern "C" int tlie_rope_cache(const void* qkv, int in_dtype, int nsplit, long long split_stride,
                                const int* positions, const int* slot_map, const float* inv_freq, int rot_dim,
                                void* q_out, void* cache, int act_dtype, int tokens, int nq, int nkv, int d,
-                               int page_size, void* stream) {
+                               int page_size, int paired, void* stream) {
   if (tokens <= 0 || nq <= 0 || nkv <= 0 || d <= 0 || d > 1024 || page_size <= 0 || nsplit < 1) return kBadArgument;
   if (rot_dim < 0 || rot_dim > d || rot_dim % 2 != 0) return kBadArgument;
   const int heads = nq + 2 * nkv;
@@ -92,7 +97,7 @@ extern "C" int tlie_rope_cache(const void* qkv, int in_dtype, int nsplit, long l
   if (in_dtype == DC && act_dtype == AC) {                                                                   \
     hipLaunchKernelGGL((rope_cache_kernel<D, A>), grid, dim3(threads), lds, s, (const D*)qkv, nsplit,         \
                        (size_t)split_stride, positions, slot_map, inv_freq, rot_dim, (A*)q_out, (A*)cache, nq, \
-                       nkv, d, page_size);                                                                   \
+                       nkv, d, page_size, paired);                                                           \
     return launch_status();                                                                                  \
   }
   TLIE_CASE(kF32, float, kF32, float)

@@ -165,10 +165,27 @@ def _check_cache(cache: torch.Tensor, num_kv_heads: int, head_dim: int, what: st
     return cache.shape[3] // head_dim
 
 
+def paired_rows(num_heads: int, num_kv_heads: int, head_dim: int, rot_dim: int) -> torch.Tensor:
+    """The order in which the rows of a fused q/k/v weight are stored when rotation pairs are to sit
+    side by side: within each q and k head, element i of the rotated part goes to 2i and element
+    i + rot_dim / 2 to 2i + 1; everything else stays.  Returns the source row of each stored row."""
+    half = rot_dim // 2
+    inside = []
+    for i in range(half):
+        inside += [i, i + half]
+    inside += list(range(rot_dim, head_dim))
+    order = []
+    for head in range(num_heads + num_kv_heads):
+        order += [head * head_dim + e for e in inside]
+    order += list(range((num_heads + num_kv_heads) * head_dim, (num_heads + 2 * num_kv_heads) * head_dim))
+    return torch.tensor(order, dtype=torch.long)
+
+
 def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, inv_freq: torch.Tensor | None,
                rot_dim: int, cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-               act_dtype: torch.dtype) -> torch.Tensor:
+               act_dtype: torch.dtype, paired: bool = False) -> torch.Tensor:
     """Rotates q and k, returns q [T, nq * d], writes k and v into the cache rows of `slot_map`.
+    paired: qkv's columns are in the order of `paired_rows`.
 
     slot_map[t] = page * page_size + row, or -1 to skip.  The slot map comes from the cache
     manager, which hands out only rows of pages it owns."""
@@ -192,7 +209,7 @@ def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, in
     _check(library().tlie_rope_cache(_ptr(qkv.data), dtype_code(qkv.data.dtype), qkv.nsplit,
                                      ctypes.c_longlong(qkv.split_stride), _ptr(positions), _ptr(slot_map), _ptr(inv_freq),
                                      rot_dim, _ptr(q_out), _ptr(cache), dtype_code(act_dtype), tokens, num_heads,
-                                     num_kv_heads, head_dim, page_size, _stream()), "rope_cache")
+                                     num_kv_heads, head_dim, page_size, 1 if paired else 0, _stream()), "rope_cache")
     return q_out
 
 
@@ -432,14 +449,29 @@ def gemm_rows_shape(out_features: int, in_features: int) -> tuple[int, int]:
     return waves, rows_per_block
 
 
+@dataclass
+class RopeTarget:
+    """What the rotation and cache write need besides the q/k/v product: see `rope_cache`."""
+    positions: torch.Tensor
+    slot_map: torch.Tensor
+    inv_freq: torch.Tensor | None
+    rot_dim: int
+    cache: torch.Tensor
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+
+
 def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str = "store",
               residual: torch.Tensor | None = None, next_norm: tuple | None = None, waves: int | None = None,
-              rows_per_block: int | None = None):
+              rows_per_block: int | None = None, rope: RopeTarget | None = None):
     """y = x . W^T (+ bias) for at most 16 rows.  x: bfloat16 [M, K], or `NormedRows` (then the
     result's rows are scaled as the norm would have scaled the input).
     epilogue "store": float32 [M, N] as a `Product`.  "silu": W's rows alternate gate and up;
     returns bfloat16 silu(gate) * up [M, N / 2].  "residual": residual [M, N] += y in place, returns
-    a `ResidualUpdated`, with the next norm's inputs when next_norm = (weight [N], eps) is given."""
+    a `ResidualUpdated`, with the next norm's inputs when next_norm = (weight [N], eps) is given.
+    "rope": W is a fused q/k/v weight with rows in the order of `paired_rows`; q and k are rotated,
+    k and v written to the cache (as `rope_cache` does), bfloat16 q [M, nq * d] is returned."""
     scale = x if isinstance(x, NormedRows) else None
     data = scale.xg if scale is not None else x
     _device_tensor(data, "x", torch.bfloat16)
@@ -487,12 +519,39 @@ def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str 
             next_code = dtype_code(next_weight.dtype)
             xg = torch.empty((rows, out_features), dtype=torch.bfloat16, device=device)
             ssq_out = torch.empty(((out_features + rows_per_block - 1) // rows_per_block, 16), dtype=torch.float32, device=device)
+    elif epilogue == "rope":
+        code = 3
+        if rope is None:
+            raise invalid_argument("gemm_rows: the rotation epilogue needs a RopeTarget")
+        _device_tensor(rope.positions, "positions", torch.int32)
+        _device_tensor(rope.slot_map, "slot_map", torch.int32)
+        _device_tensor(rope.cache, "cache", torch.bfloat16)
+        if out_features != (rope.num_heads + 2 * rope.num_kv_heads) * rope.head_dim:
+            raise invalid_shape(f"gemm_rows: {out_features} rows of W are not (nq + 2 nkv) * d")
+        if rope.positions.shape != (rows,) or rope.slot_map.shape != (rows,):
+            raise invalid_shape("gemm_rows: positions and slot_map need one entry per token")
+        page_size = _check_cache(rope.cache, rope.num_kv_heads, rope.head_dim, "gemm_rows")
+        rot_dim = rope.rot_dim if rope.inv_freq is not None else 0
+        if rope.inv_freq is not None:
+            _device_tensor(rope.inv_freq, "inv_freq", torch.float32)
+            if rot_dim % 2 != 0 or not 0 < rot_dim <= rope.head_dim or rope.inv_freq.shape != (rot_dim // 2,):
+                raise invalid_shape("gemm_rows: inv_freq needs rot_dim / 2 entries, rot_dim even and at most d")
+        if rope.head_dim % 2 != 0:
+            raise invalid_shape("gemm_rows: the rotation epilogue needs an even head size")
+        q_out = torch.empty((rows, rope.num_heads * rope.head_dim), dtype=torch.bfloat16, device=device)
     else:
         raise invalid_argument(f"gemm_rows: unknown epilogue '{epilogue}'")
+    if rope is None or epilogue != "rope":
+        rope_args = (_ptr(None), _ptr(None), _ptr(None), 0, 0, 0, 0, 0, _ptr(None), _ptr(None))
+    else:
+        rope_args = (_ptr(rope.positions), _ptr(rope.slot_map), _ptr(rope.inv_freq), rot_dim, rope.num_heads,
+                     rope.num_kv_heads, rope.head_dim, page_size, _ptr(q_out), _ptr(rope.cache))
     _check(library().tlie_gemm_rows(_ptr(data), _ptr(weight), _ptr(bias), rows, out_features, in_features, _ptr(ssq_in),
                                     strips_in, in_features, ctypes.c_float(eps), code, _ptr(y), _ptr(act), _ptr(residual),
-                                    _ptr(next_weight), next_code, _ptr(xg), _ptr(ssq_out), waves, rows_per_block, _stream()),
-           "gemm_rows")
+                                    _ptr(next_weight), next_code, _ptr(xg), _ptr(ssq_out), *rope_args, waves, rows_per_block,
+                                    _stream()), "gemm_rows")
+    if epilogue == "rope":
+        return q_out
     if epilogue == "store":
         return Product(y, 1)
     if epilogue == "silu":

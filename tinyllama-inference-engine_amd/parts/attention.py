@@ -55,8 +55,16 @@ class Attention(Mixer):
         return specs
 
     def load(self, weights, prefix):
+        # The rows of the fused q/k/v weight are stored with the two elements of a rotation pair
+        # side by side when the position encoding is a rotation table: the product of few rows then
+        # rotates and writes the cache itself; the kernels that read its output know the order.
+        table = self.position.rotary_table()
+        self.paired = table is not None
+        order = ops.paired_rows(self.nq, self.nkv, self.d, table[1]).to(self.device) if self.paired else None
+
         def cat(suffix):
-            return torch.cat([weights[f"{prefix}{name}_proj.{suffix}"] for name in "qkv"], dim=0)
+            joined = torch.cat([weights[f"{prefix}{name}_proj.{suffix}"] for name in "qkv"], dim=0)
+            return joined[order].contiguous() if order is not None else joined
         self.qkv = Linear(cat("weight"), cat("bias") if self.bias else None, self.dtype)
         self.o = Linear(weights[prefix + "o_proj.weight"], weights.get(prefix + "o_proj.bias") if self.bias else None,
                         self.dtype)
@@ -76,14 +84,19 @@ class Attention(Mixer):
 
     def forward(self, x, ctx, binding: Binding, into=None):
         pages = ctx.groups[binding.group]
-        qkv = self.qkv(x)
         slot_map = pages.slot_map if binding.writes else ctx.no_slots
         table = self.position.rotary_table()
-        if table is None and type(self.position).apply_qk is not PositionEncoding.apply_qk:
-            qkv = self._apply_other_positions(qkv, ctx)
         inv_freq, rot_dim = table if table is not None else (None, 0)
-        q = ops.rope_cache(qkv, ctx.positions, slot_map, inv_freq, rot_dim, binding.cache, self.nq, self.nkv, self.d,
-                           self.dtype)
+        other_positions = table is None and type(self.position).apply_qk is not PositionEncoding.apply_qk
+        target = None
+        if not other_positions:
+            target = ops.RopeTarget(ctx.positions, slot_map, inv_freq, rot_dim, binding.cache, self.nq, self.nkv, self.d)
+        q = self.qkv(x, rope=target)
+        if isinstance(q, ops.Product):              # the product did not rotate: a kernel of its own does
+            if other_positions:
+                q = self._apply_other_positions(q, ctx)
+            q = ops.rope_cache(q, ctx.positions, slot_map, inv_freq, rot_dim, binding.cache, self.nq, self.nkv, self.d,
+                               self.dtype, paired=self.paired)
         page_size = binding.cache.shape[3] // self.d
         if ops.attention_mfma_takes(self.dtype, self.d, page_size):
             tiles, col_tiles, nsplit, split_len = ctx.attention_tiles(self.nq // self.nkv, self.nkv, self.d)

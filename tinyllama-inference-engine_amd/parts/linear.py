@@ -33,20 +33,25 @@ class Linear:
         ask for the gate, or for the add into the residual)."""
         return ops.gemm_rows_takes(rows, self.weight, self.dtype)
 
-    def __call__(self, x, out_dtype: torch.dtype | None = None, whole: bool = False, into=None, gated: bool = False):
+    def __call__(self, x, out_dtype: torch.dtype | None = None, whole: bool = False, into=None, gated: bool = False,
+                 rope=None):
         """out_dtype: what a dense result is stored in (the skinny kernel's partial sums are float32
         whatever it says).  whole: the caller has no kernel that adds partial sums up, so the
         product must come as one array (the skinny kernel then does not split K).
         into (a `ResidualTarget`): add the result into the residual, if the kernel for this step can
         (then a `ResidualUpdated` comes back, else the result as usual).  gated: the weight's rows
         alternate gate and up; if the kernel for this step can, silu(gate) * up comes back as a
-        tensor, else the product as usual."""
+        tensor, else the product as usual.  rope (an `ops.RopeTarget`; the weight's rows are in
+        paired order): if the kernel for this step can, q and k are rotated, k and v written to the
+        cache and q comes back as a tensor, else the product as usual."""
         out_dtype = out_dtype or self.dtype
         if self.takes_rows(x.shape[0]):
             if into is not None:
                 return ops.gemm_rows(x, self.weight, self.bias, "residual", residual=into.residual, next_norm=into.next_norm)
             if gated:
                 return ops.gemm_rows(x, self.weight, self.bias, "silu")
+            if rope is not None:
+                return ops.gemm_rows(x, self.weight, self.bias, "rope", rope=rope)
             if isinstance(x, ops.NormedRows):
                 return ops.gemm_rows(x, self.weight, self.bias, "store")
         if isinstance(x, ops.NormedRows):
