@@ -344,6 +344,13 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
         decode = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
                                     1.0 / math.sqrt(d), nsplit, split_len)
         assert torch.equal(decode, out)
+        # several waves of a workgroup sharing the keys: the same result within rounding (the sums run in another order)
+        waves = 2
+        while waves <= 16 and waves * d <= 1024:
+            shared = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
+                                        1.0 / math.sqrt(d), nsplit, split_len, 1, waves)
+            assert rel_err(shared, out.double()) < 1e-2, f"{waves} waves"
+            waves *= 2
     return out.view(len(token_list), nq, d)
 
 

@@ -22,10 +22,11 @@
 //  * Keys are walked in blocks of 32 that start at multiples of 32 from position 0, with a running
 //    maximum and sum: the context length is unbounded and the order of the sums for a (sequence,
 //    position) does not depend on how the step was cut.
-//  * With nsplit > 1 the keys are cut into nsplit parts of split_len positions handled by
-//    different waves (a decode step of few sequences would otherwise leave most of the chip idle);
-//    each writes an unnormalised partial result with its maximum and sum, and a second kernel
-//    merges them.  The parts are fixed ranges of positions, so a wave can fetch its first keys
+//  * A decode step of few sequences has few tiles, so the keys of a tile are shared out.  First
+//    among the waves of a workgroup (up to 16): wave w takes the blocks w, w + W, ... and the
+//    waves' results are merged through LDS, so the kernel still writes final results.  Then, for
+//    long contexts, among nsplit workgroups of split_len positions each, which write unnormalised
+//    partial results with their maxima and sums for a second kernel to merge.  The parts are fixed ranges of positions, so a wave can fetch its first keys
 //    before it knows how long the sequence is: the position, the block table and the keys are not
 //    three loads in a row.
 #include "common.h"
@@ -79,8 +80,10 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // sequence * ceil(G / 16) + tile of the group.
 // DT = head_dim / 16.  CT = groups of 16 columns per wave: a tile has 16 * CT columns, and every
 // key and value the wave loads serves all of them (prompt portions take CT = 4, decode steps 1).
+// A workgroup has at most 1024 / (16 * CT * DT) waves (16 at most): their merge fits LDS, and the
+// compiler may give each wave the registers that leaves.
 template <int DT, int CT>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(64 * (1024 / (16 * CT * DT) > 16 ? 16 : (1024 / (16 * CT * DT) < 1 ? 1 : 1024 / (16 * CT * DT))))
 attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache,
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
@@ -89,6 +92,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;                 // 32-wide k steps of the first product
   const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
+  const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;     // waves that share the tile's keys
   const int kvh = blockIdx.y, split = blockIdx.z;
   // whether a lane's 8 dims of k step ks exist: always, unless the head size is an odd multiple of 16
   auto has_dims = [&](int ks) { return DT % 2 == 0 || ks < KS - 1 || grp < 2; };
@@ -290,7 +294,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
 
   // Two blocks in turn: while one is worked on, the other is on its way.  Without a window the
   // first block's place is known before the position is: split_lo & ~31.
-  const int first_block = (window > 0 ? range_lo : split_lo) & ~31;
+  const int first_block = ((window > 0 ? range_lo : split_lo) & ~31) + 32 * wave;
+  const int stride = 32 * waves;
   // a block that every column of the tile sees whole: inside the range, below the first column's
   // position, inside the last column's window
   const int open_lo = max((range_lo + 31) & ~31, window > 0 ? tile_hi - window : 0);
@@ -303,15 +308,70 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   };
   KeyBlock even, odd;
   load_block(first_block, even);
-  for (int kb = first_block; kb < range_hi; kb += 64) {
-    load_block(kb + 32, odd);
+  for (int kb = first_block; kb < range_hi; kb += 2 * stride) {
+    load_block(kb + stride, odd);
     work(kb, even);
-    if (kb + 32 >= range_hi) break;
-    load_block(kb + 64, even);
-    work(kb + 32, odd);
+    if (kb + stride >= range_hi) break;
+    load_block(kb + 2 * stride, even);
+    work(kb + stride, odd);
   }
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) running_sum[ct] = groups_sum(running_sum[ct]);
+
+  if (waves > 1) {
+    // ---- the waves' results into one, through LDS -------------------------------------------------
+    extern __shared__ float lds[];
+    float* stats = lds;                                  // [waves][CT][16][2]: maximum, sum
+    float* slots = lds + waves * CT * 32;                // [waves / 2][CT * DT][64][4]
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+      if (grp == 0) {
+        stats[((wave * CT + ct) * 16 + col) * 2] = running_max[ct];
+        stats[((wave * CT + ct) * 16 + col) * 2 + 1] = running_sum[ct];
+      }
+    __syncthreads();
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      float top = -INFINITY;
+      for (int w = 0; w < waves; ++w) top = fmaxf(top, stats[((w * CT + ct) * 16 + col) * 2]);
+      float total = 0.f;
+      for (int w = 0; w < waves; ++w) {
+        const float m = stats[((w * CT + ct) * 16 + col) * 2];
+        if (m != -INFINITY) total += __builtin_amdgcn_exp2f(m - top) * stats[((w * CT + ct) * 16 + col) * 2 + 1];
+      }
+      const float mine = running_max[ct] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(running_max[ct] - top);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) o[ct][dt][j] *= mine;
+      running_max[ct] = top;
+      running_sum[ct] = total;
+    }
+    // all results are now on the same scale: add them pairwise, the upper half of the waves handing
+    // theirs to the lower half, until wave 0 holds the sum
+    for (int half = waves >> 1; half >= 1; half >>= 1) {
+      __syncthreads();
+      if (wave >= half && wave < 2 * half) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<float4*>(slots + (((wave - half) * CT * DT + ct * DT + dt) * 64 + lane) * 4) =
+                make_float4(o[ct][dt][0], o[ct][dt][1], o[ct][dt][2], o[ct][dt][3]);
+      }
+      __syncthreads();
+      if (wave < half) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+          for (int dt = 0; dt < DT; ++dt) {
+            const float4 other = *reinterpret_cast<const float4*>(slots + ((wave * CT * DT + ct * DT + dt) * 64 + lane) * 4);
+            o[ct][dt][0] += other.x, o[ct][dt][1] += other.y, o[ct][dt][2] += other.z, o[ct][dt][3] += other.w;
+          }
+      }
+    }
+    if (wave != 0) return;
+  }
 
   // o[ct][dt][j] is dim dt*16 + grp*4 + j of the column; maxima and sums are in base 2
 #pragma unroll
@@ -382,9 +442,13 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
 template <int DT, int CT>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
-                            int split_len, int nq, int nkv, int page_size, int window, float scale, hipStream_t stream) {
+                            int split_len, int nq, int nkv, int page_size, int window, float scale, int waves,
+                            hipStream_t stream) {
   const float scale_log2 = scale * 1.4426950408889634f;
-  hipLaunchKernelGGL((attention_mfma_kernel<DT, CT>), dim3(num_tiles, nkv, nsplit), dim3(64), 0, stream, (const uint16_t*)q,
+  // LDS for merging the waves: their maxima and sums, and half as many slots as waves for the results
+  const size_t lds = waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
+  if (lds > 64 * 1024) return kBadArgument;
+  hipLaunchKernelGGL((attention_mfma_kernel<DT, CT>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                      (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
                      part_ml, nsplit, split_len, nq, nkv, page_size, window, scale_log2);
   return launch_status();
@@ -400,20 +464,22 @@ using namespace tlie;
 // part_o: float [tokens * nq * nsplit * d], part_ml: float [tokens * nq * nsplit * 2] (both only when nsplit > 1);
 // split_len: positions per part, a multiple of 32, nsplit * split_len >= the longest sequence.
 // d % 16 == 0, d <= 256, page_size a power of two >= 16; col_tiles 1, or 4 for d <= 64, or 2 for d <= 128.
+// waves: 1, 2, 4, 8 or 16 waves of a workgroup share a tile's keys; waves * col_tiles * d <= 1024 (their merge's LDS).
 extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
                                    const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                                    float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
-                                   int d, int page_size, int window, float scale, void* stream) {
+                                   int d, int page_size, int window, float scale, int waves, void* stream) {
   if (num_tiles <= 0 || tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || d % 16 != 0 ||
       page_size < 16 || (page_size & (page_size - 1)) != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
     return kBadArgument;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr || split_len <= 0 || split_len % 32 != 0)) return kBadArgument;
   if (col_tiles != 1 && !(col_tiles == 4 && d <= 64) && !(col_tiles == 2 && d <= 128)) return kBadArgument;
+  if (waves < 1 || waves > 16 || (waves & (waves - 1)) != 0 || (waves > 1 && waves * col_tiles * d > 1024)) return kBadArgument;
   if (tiles == nullptr && (col_tiles != 1 || num_tiles != tokens * ((nq / nkv + 15) / 16))) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
   int status = kBadArgument;
 #define TLIE_ARGS q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, nsplit, split_len, nq, \
-                  nkv, page_size, window, scale, s
+                  nkv, page_size, window, scale, waves, s
 #define TLIE_CASE(DT)                                        \
   case DT:                                                   \
     status = launch_attention<DT, 1>(TLIE_ARGS);             \

@@ -64,7 +64,7 @@ class StepContext:
         as many parts as it takes to give a step of few tiles about a thousand waves (measured: at
         batch 64 and 2048 positions 4 parts reach 5 TB/s, 16 parts 4 TB/s, and merging more than 16
         costs more than it gains), each part a multiple of 32 positions and at least 64.
-        Returns (tiles, col_tiles, nsplit, split_len)."""
+        Returns (tiles, col_tiles, nsplit, split_len, waves of a workgroup that share a tile's keys)."""
         decode = self.max_new == 1 and self.num_seqs == self.num_tokens
         col_tiles = 1
         if decode:
@@ -77,15 +77,24 @@ class StepContext:
                 self._tiles[(groups_per_kv, col_tiles)] = torch.from_numpy(tiles).to(self.tokens.device)
             tiles = self._tiles[(groups_per_kv, col_tiles)]
             count = tiles.shape[0]
-        waves = count * num_kv_heads
-        # a step of prompt portions has tiles enough; cutting their keys would only add merging
-        target = 1024 if decode else 512
-        nsplit = max(1, min((target + waves - 1) // waves, 16, (self.max_context + 63) // 64))
+        tiles_all = count * num_kv_heads
+        if not decode:
+            # a step of prompt portions has tiles enough; cutting their keys would only add merging
+            nsplit, waves = max(1, min((512 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64)), 1
+        else:
+            # workgroups share a tile's keys until there is one for every compute unit (their sums
+            # meet in the merge kernel); then the waves of a workgroup share them, which costs no
+            # launch, while a wave keeps 128 keys or more
+            nsplit = max(1, min((256 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
+            waves = 1
+            while (waves < 4 and waves * 2 * head_dim <= 1024 and tiles_all * nsplit * waves * 2 <= 1024
+                   and self.max_context >= nsplit * waves * 2 * 128):
+                waves *= 2
         if nsplit == 1:
-            return tiles, col_tiles, 1, 0
+            return tiles, col_tiles, 1, 0, waves
         split_len = ((self.max_context + nsplit - 1) // nsplit + 31) // 32 * 32
         nsplit = (self.max_context + split_len - 1) // split_len
-        return tiles, col_tiles, nsplit, split_len
+        return tiles, col_tiles, nsplit, split_len, waves
 
 
 class ModelRunner:

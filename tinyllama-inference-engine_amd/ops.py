@@ -358,7 +358,7 @@ def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> b
 
 def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor | None,
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
-                   scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1) -> torch.Tensor:
+                   scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1, waves: int = 1) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
@@ -366,7 +366,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     a decode step, in which token i is the one token of sequence i.  nsplit > 1 cuts the keys into
     that many parts of split_len positions (a multiple of 32; nsplit * split_len must reach the
     longest sequence) that run side by side and are merged.  col_tiles: the value the tiles were
-    made with."""
+    made with.  waves (a power of two up to 16, waves * col_tiles * d <= 1024): so many waves of a
+    workgroup share each tile's (or part's) keys and merge their results before writing."""
     _device_tensor(q, "q", torch.bfloat16)
     _device_tensor(cache, "cache", torch.bfloat16)
     _device_tensor(block_table, "block_table", torch.int32)
@@ -393,6 +394,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
         num_tiles = tokens * ((num_heads // num_kv_heads + 15) // 16)
     if nsplit > 1 and (split_len <= 0 or split_len % 32 != 0):
         raise invalid_argument("attention: split_len must be a positive multiple of 32")
+    if waves not in (1, 2, 4, 8, 16) or (waves > 1 and waves * col_tiles * head_dim > 1024):
+        raise invalid_argument("attention: waves must be a power of two up to 16 with waves * col_tiles * d <= 1024")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
         raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a power of two of rows (at least 16)")
     out = torch.empty_like(q)
@@ -403,7 +406,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
                                          num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
                                          split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
-                                         int(window) if window else 0, ctypes.c_float(scale), _stream()), "attention_mfma")
+                                         int(window) if window else 0, ctypes.c_float(scale), waves, _stream()),
+           "attention_mfma")
     return out
 
 
