@@ -291,3 +291,51 @@ def test_replay_program_and_command_line(setups, tmp_path):
     assert run.returncode != 0 and error_code(run.stderr) == "tokenizer_error"
     run = subprocess.run(cli + ["generate", setup["folder"], prompt, "200"], capture_output=True, text=True, timeout=300)
     assert run.returncode != 0 and error_code(run.stderr) == "out_of_bounds"         # app/reference_cli.cpp:72-75
+
+
+# The layer sizes that the benchmark runs (width 2048, 32 heads on 4 groups of size 64, feed-forward
+# 5632, vocabulary 32000), with two layers: the kernels' variants for these sizes (row products of 16
+# rows at 2048 and 5632 columns, 8 query heads a key head, split keys, recorded steps) are the ones a
+# served model runs, and the tiny configurations reach other variants.
+BENCH_SHAPE = dict(model_type="llama", architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=5632,
+                   num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=4, max_position_embeddings=2048,
+                   vocab_size=32000, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False,
+                   attention_bias=False, hidden_act="silu", bos_token_id=1, eos_token_id=2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_benchmark_layer_sizes_cut_three_ways(tmp_path, dtype):
+    folder = make_model(tmp_path / "model", BENCH_SHAPE, seed=5, dtype_name=dtype, std=0.02, norm_std=0.1)
+    raw, weights = load_plain(folder)
+    length = 300
+    tokens = random_tokens(77, length, BENCH_SHAPE["vocab_size"])
+    want = plain_forward(raw, weights, tokens)
+    del weights
+    from tlie_amd import Engine
+    engine = Engine(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4)
+    whole = Replayer(engine)
+    whole.step([("w", tokens, list(range(length)))], end=["w"])
+    bad = first_bad_row(whole.logits_of("w", range(length)), want, TOLERANCE[dtype])
+    assert bad is None, f"whole prompt: first wrong position {bad}"
+    # most in one step, the last 32 one by one, beside a second request that decodes the same tokens
+    cut = Replayer(engine)
+    cut.step([("a", tokens[:length - 32], []), ("b", tokens[:length - 32], [])])
+    for position in range(length - 32, length):
+        cut.step([("a", [tokens[position]], [0]), ("b", [tokens[position]], [0])])
+    engine.finish("a")
+    engine.finish("b")
+    for request in "ab":
+        got = cut.logits_of(request, range(length - 32, length))
+        bad = first_bad_row(got, want[length - 32:], TOLERANCE[dtype])
+        assert bad is None, f"decoded position {length - 32 + bad} of {request} is wrong"
+    # portions of changing size, down to two tokens
+    portions = Replayer(engine)
+    sizes, cursor, turn = [100, 2, 16, 3, 64, 17, 5, 1, 33], 0, 0
+    while cursor < length:
+        size = min(sizes[turn % len(sizes)], length - cursor)
+        portions.step([("p", tokens[cursor:cursor + size], list(range(size)))])
+        cursor += size
+        turn += 1
+    engine.finish("p")
+    bad = first_bad_row(portions.logits_of("p", range(length)), want, TOLERANCE[dtype])
+    assert bad is None, f"portions {sizes}: first wrong position {bad}"

@@ -320,8 +320,9 @@ def test_gemm_skinny_refuses():
     assert not ops.gemm_skinny_takes(torch.randn(2, 12, device=DEV).bfloat16(), torch.randn(8, 12, device=DEV).bfloat16())
 
 
-def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0, col_tiles=None):
-    """One sequence through the tiled kernel: q rows for the positions in token_list (default all)."""
+def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0, col_tiles=None, waves=1):
+    """One sequence through the tiled kernel: q rows for the positions in token_list (default all).
+    waves > 1: so many waves share each tile's keys, and the tiles come longest first."""
     from tlie_amd import ops
     import numpy as np
     tokens, nq, d = q.shape
@@ -332,14 +333,17 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     assert token_list == list(range(token_list[0], token_list[0] + len(token_list)))
     table = torch.tensor([[0] * len(pages), pages], dtype=torch.int32, device=DEV)
     col_tiles = col_tiles or ops.attention_col_tiles(d)
-    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv, col_tiles)
+    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv, col_tiles,
+                                np.asarray([token_list[-1] + 1]) if waves > 1 else None)
+    if waves > 1 and tiles.shape[0] > 1:
+        assert tiles[0, 3] > tiles[-1, 3]                                      # the tile of the last tokens first
     tiles[:, 0] = 1                                                            # the sequence is row 1 of the table
     split_len = ((tokens + nsplit - 1) // nsplit + 31) // 32 * 32
     rows = q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV)
     positions = torch.tensor(token_list, dtype=torch.int32, device=DEV)
     out = ops.attention_mfma(rows, cache.to(DEV), table, torch.from_numpy(tiles).to(DEV), positions, nq, nkv, d, window,
-                             1.0 / math.sqrt(d), nsplit, split_len, col_tiles)
-    if len(token_list) == 1:
+                             1.0 / math.sqrt(d), nsplit, split_len, col_tiles, waves)
+    if len(token_list) == 1 and waves == 1:
         # the same step as a decode step: no work list, the kernel derives the tiles; the sequence must be row 0
         decode = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
                                     1.0 / math.sqrt(d), nsplit, split_len)
@@ -373,8 +377,16 @@ def test_attention_mfma(case):
     want = plain_attention(rounded(q, torch.bfloat16), rounded(k, torch.bfloat16), rounded(v, torch.bfloat16), window=window)
     whole = run_attention_mfma(q, k, v, page, window, 1, shuffle_seed=tokens)
     assert rel_err(whole, want) < TOL["bfloat16"]
-    narrow = run_attention_mfma(q, k, v, page, window, 1, shuffle_seed=tokens, col_tiles=1)       # 16 columns a wave
-    assert rel_err(narrow, want) < TOL["bfloat16"]
+    for col_tiles in (1, 2, 4):                                   # 16, 32, 64 columns a wave, where the head size allows
+        if col_tiles * d <= 256:
+            narrow = run_attention_mfma(q, k, v, page, window, 1, shuffle_seed=tokens, col_tiles=col_tiles)
+            assert rel_err(narrow, want) < TOL["bfloat16"], f"{col_tiles} column groups"
+    # 2 and 4 waves of a workgroup share each tile's keys (whole and in 3 parts), the tiles longest first
+    for waves, nsplit in ((2, 1), (4, 1), (4, 3)):
+        col_tiles = 2 if d <= 128 else 1
+        if waves * col_tiles * d <= 1024:
+            shared = run_attention_mfma(q, k, v, page, window, nsplit, shuffle_seed=tokens, col_tiles=col_tiles, waves=waves)
+            assert rel_err(shared, want) < TOL["bfloat16"], f"{waves} waves, {nsplit} parts"
     # the last token alone (a decode step), its key range cut in parts that are merged
     for nsplit in (1, 2, 5):
         last = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=tokens)

@@ -38,8 +38,6 @@ namespace tlie {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
-typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
 
 union Pack8 {
   uint4 u;
@@ -65,12 +63,6 @@ __device__ __forceinline__ float groups_sum(float v) {
   v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
   r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
-// two floats to two bfloat16 (round to nearest even) in one instruction, v_cvt_pk_bf16_f32
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  const bf16x2 r = __builtin_convertvector((floatx2{lo, hi}), bf16x2);
-  return *reinterpret_cast<const uint32_t*>(&r);
 }
 
 // tiles[i] = (sequence row of the block table, index of the sequence's first token in this step,
@@ -228,7 +220,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
         for (int ks = 0; ks < KS; ++ks)
           s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(block.k[t][ks].v, qreg[ct][ks].v, s[ct][t], 0, 0, 0);
       }
-    // ---- mask, scale, maximum: s[ct][t][j] is key kb + t*16 + grp*4 + j of the column --------------
+    // ---- mask and maximum (the scale goes into the exponent's multiply-add): s[ct][t][j] is key kb + t*16 + grp*4 + j of the column --------------
     float block_max[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
@@ -240,15 +232,13 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
           if (kMasked) {
             const int key = kb + t * 16 + grp * 4 + j;
             const bool ok = key >= range_lo && key < range_hi && key <= pos_col[ct] && key >= lo_col[ct];
-            s[ct][t][j] = ok ? s[ct][t][j] * scale_log2 : -INFINITY;
-          } else {
-            s[ct][t][j] *= scale_log2;
+            s[ct][t][j] = ok ? s[ct][t][j] : -INFINITY;
           }
           block_max[ct] = fmaxf(block_max[ct], s[ct][t][j]);
         }
     }
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) block_max[ct] = groups_max(block_max[ct]);
+    for (int ct = 0; ct < CT; ++ct) block_max[ct] = groups_max(block_max[ct]) * scale_log2;   // the scale is positive
     // ---- running softmax: the column's four lane groups share the maximum, so each keeps the sum of
     // its own keys and the groups' sums are added once, after the last block ------------------------
     float alpha[CT];
@@ -266,7 +256,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) e[t * 4 + j] = __builtin_amdgcn_exp2f(s[ct][t][j] - new_max);   // 0 for masked keys
+          for (int j = 0; j < 4; ++j) e[t * 4 + j] = __builtin_amdgcn_exp2f(fmaf(s[ct][t][j], scale_log2, -new_max));   // 0 for masked keys
         running_sum[ct] = running_sum[ct] * alpha[ct] + (((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7])));
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[ct].w[i] = pack_bf16(e[2 * i], e[2 * i + 1]);
@@ -476,6 +466,7 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   if (col_tiles != 1 && !(col_tiles == 4 && d <= 64) && !(col_tiles == 2 && d <= 128)) return kBadArgument;
   if (waves < 1 || waves > 16 || (waves & (waves - 1)) != 0 || (waves > 1 && waves * col_tiles * d > 1024)) return kBadArgument;
   if (tiles == nullptr && (col_tiles != 1 || num_tiles != tokens * ((nq / nkv + 15) / 16))) return kBadArgument;
+  if (!(scale > 0.f)) return kBadArgument;     // the maximum is taken before the scores are scaled
   hipStream_t s = (hipStream_t)stream;
   int status = kBadArgument;
 #define TLIE_ARGS q, cache, block_table, max_blocks, tiles, num_tiles, positions, out, part_o, part_ml, nsplit, split_len, nq, \

@@ -50,6 +50,46 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const D* __rest
   }
 }
 
+// The same with eight elements a thread (16-byte loads and stores): hidden % 8 == 0, one summand.
+template <typename D, typename W, typename O>
+__global__ void add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* __restrict__ delta,
+                                        const W* __restrict__ weight, float eps, O* __restrict__ out,
+                                        const int* __restrict__ rows, int hidden) {
+  extern __shared__ float row_cache[];           // hidden floats, then 16 for the reduction
+  float* scratch = row_cache + hidden;
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* res = residual + static_cast<size_t>(src) * hidden;
+  float square = 0.f;
+  for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+    float v[8];
+    load8(res + i, v);
+    if (delta) {
+      float d[8];
+      load8(delta + static_cast<size_t>(src) * hidden + i, d);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] += d[j];
+      if (!rows) store8(res + i, v);
+    }
+    store8(row_cache + i, v);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) square += v[j] * v[j];
+  }
+  const float total = block_sum(square, scratch);
+  const float scale = rsqrtf(total / static_cast<float>(hidden) + eps);
+  if (out) {
+    O* o = out + static_cast<size_t>(r) * hidden;
+    for (int i = threadIdx.x * 8; i < hidden; i += blockDim.x * 8) {
+      float v[8], w[8];
+      load8(row_cache + i, v);                   // the thread's own entries
+      load8(weight + i, w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = v[j] * scale * w[j];
+      store8(o + i, v);
+    }
+  }
+}
+
 // ---- act[t, i] = silu(gate[t, i]) * up[t, i]; gate_up is [rows, 2 * inter], either [gate | up] or,
 // interleaved, g0 u0 g1 u1 ... (the layout the gated product of few rows wants of its weight) -------
 // reference: (g / (1 + exp(-g))) * u in float (src/cuda/kernels.cu:198-206)
@@ -64,6 +104,36 @@ __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_
     const float g = sum_splits(base + (interleaved ? 2 * i : i), nsplit, split_stride);
     const float u = sum_splits(base + (interleaved ? 2 * i + 1 : inter + i), nsplit, split_stride);
     out[index] = from_float<O>((g / (1.f + expf(-g))) * u);
+  }
+}
+
+// Eight results a thread from sixteen inputs: inter % 8 == 0, one summand.
+template <typename D, typename O>
+__global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, O* __restrict__ out, int rows, int inter,
+                                     int interleaved) {
+  const int per_row = inter / 8;
+  const size_t total = static_cast<size_t>(rows) * per_row;
+  for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
+       index += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    const size_t t = index / per_row;
+    const int i = static_cast<int>(index % per_row) * 8;
+    const D* base = gate_up + t * 2 * inter;
+    float a[8], b[8], g[8], u[8];
+    if (interleaved) {
+      load8(base + 2 * i, a);
+      load8(base + 2 * i + 8, b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        g[j] = a[2 * j]; u[j] = a[2 * j + 1];
+        g[4 + j] = b[2 * j]; u[4 + j] = b[2 * j + 1];
+      }
+    } else {
+      load8(base + i, g);
+      load8(base + inter + i, u);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) g[j] = (g[j] / (1.f + expf(-g[j]))) * u[j];
+    store8(out + t * inter + i, g);
   }
 }
 
@@ -90,9 +160,18 @@ template <typename D, typename W, typename O>
 static int launch_add_rmsnorm(float* residual, const void* delta, int nsplit, size_t split_stride,
                               const void* weight, float eps, void* out,
                               const int* rows, int num_rows, int hidden, hipStream_t stream) {
-  const int threads = hidden >= 2048 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
   const size_t lds = (static_cast<size_t>(hidden) + 16) * sizeof(float);
   if (lds > 160 * 1024) return kBadArgument;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(delta) |
+                         reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) & 31) == 0;
+  if ((hidden & 7) == 0 && nsplit == 1 && aligned) {
+    const int chunks = hidden / 8;
+    const int wide = chunks >= 1024 ? 1024 : (chunks + 63) / 64 * 64;
+    hipLaunchKernelGGL((add_rmsnorm_wide_kernel<D, W, O>), dim3(num_rows), dim3(wide), lds, stream, residual,
+                       (const D*)delta, (const W*)weight, eps, (O*)out, rows, hidden);
+    return launch_status();
+  }
+  const int threads = hidden >= 2048 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
   hipLaunchKernelGGL((add_rmsnorm_kernel<D, W, O>), dim3(num_rows), dim3(threads), lds, stream, residual,
                      (const D*)delta, nsplit, split_stride, (const W*)weight, eps, (O*)out, rows, hidden);
   return launch_status();
@@ -127,6 +206,23 @@ extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long
   const int threads = 256;
   const int blocks = static_cast<int>(total / threads + 1 < 65536 ? total / threads + 1 : 65536);
   hipStream_t s = (hipStream_t)stream;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(out)) & 31) == 0;
+  if ((inter & 7) == 0 && nsplit == 1 && aligned) {
+    const size_t groups = total / 8;
+    const int wide = static_cast<int>(groups / threads + 1 < 65536 ? groups / threads + 1 : 65536);
+    if (in_dtype == kF32 && out_dtype == kF32)
+      hipLaunchKernelGGL((silu_mul_wide_kernel<float, float>), dim3(wide), dim3(threads), 0, s, (const float*)gate_up,
+                         (float*)out, rows, inter, interleaved);
+    else if (in_dtype == kF32 && out_dtype == kBF16)
+      hipLaunchKernelGGL((silu_mul_wide_kernel<float, bf16>), dim3(wide), dim3(threads), 0, s, (const float*)gate_up,
+                         (bf16*)out, rows, inter, interleaved);
+    else if (in_dtype == kBF16 && out_dtype == kBF16)
+      hipLaunchKernelGGL((silu_mul_wide_kernel<bf16, bf16>), dim3(wide), dim3(threads), 0, s, (const bf16*)gate_up,
+                         (bf16*)out, rows, inter, interleaved);
+    else
+      return kBadArgument;
+    return launch_status();
+  }
   if (in_dtype == kF32 && out_dtype == kF32)
     hipLaunchKernelGGL((silu_mul_kernel<float, float>), dim3(blocks), dim3(threads), 0, s, (const float*)gate_up, nsplit,
                        (size_t)split_stride, (float*)out, rows, inter, interleaved);

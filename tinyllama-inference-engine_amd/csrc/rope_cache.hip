@@ -74,6 +74,60 @@ __global__ void rope_cache_kernel(const D* __restrict__ qkv, int nsplit, size_t 
   }
 }
 
+// The same for one summand with eight input columns a thread (16-byte loads): d % 8 == 0 and, where
+// there is rotation, paired columns and rot_dim % 8 == 0, so that a thread holds four whole pairs.
+// One block a token; blockDim.x covers (nq + 2 nkv) * d / 8 groups, or loops.
+template <typename D, typename A>
+__global__ void rope_cache_wide_kernel(const D* __restrict__ qkv, const int* __restrict__ positions,
+                                       const int* __restrict__ slot_map, const float* __restrict__ inv_freq,
+                                       int rot_dim, A* __restrict__ q_out, A* __restrict__ cache, int nq, int nkv,
+                                       int d, int page_size) {
+  extern __shared__ float lds[];
+  const int half = rot_dim / 2;
+  float* cosines = lds;                  // half
+  float* sines = cosines + half;         // half
+  const int t = blockIdx.x;
+  if (inv_freq != nullptr) {
+    const float pos = static_cast<float>(positions[t]);
+    for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
+    __syncthreads();
+  }
+  const int heads = nq + 2 * nkv, per_head = d / 8;
+  const int slot = slot_map[t];
+  const size_t head_stride = static_cast<size_t>(page_size) * d;
+  A* page = cache + static_cast<size_t>(slot < 0 ? 0 : slot / page_size) * 2 * nkv * head_stride;
+  const int row = slot < 0 ? 0 : slot % page_size;
+  for (int g = threadIdx.x; g < heads * per_head; g += blockDim.x) {
+    const int head = g / per_head, c = (g % per_head) * 8;
+    if (head >= nq && slot < 0) continue;
+    float v[8];
+    load8(qkv + (static_cast<size_t>(t) * heads + head) * d + c, v);
+    if (head >= nq + nkv) {
+      // a value head: after the nkv key heads of the page, transposed
+      A* out = page + (head - nq) * head_stride + static_cast<size_t>(c) * page_size + row;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) out[static_cast<size_t>(j) * page_size] = from_float<A>(v[j]);
+      continue;
+    }
+    A* out = head < nq ? q_out + (static_cast<size_t>(t) * nq + head) * d
+                       : page + (head - nq) * head_stride + static_cast<size_t>(row) * d;
+    if (inv_freq != nullptr && c < rot_dim) {
+      const int first = c / 2;           // v[2j], v[2j + 1] = elements first + j and first + j + half
+      float lo[4], hi[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float cs = cosines[first + j], sn = sines[first + j];
+        lo[j] = v[2 * j] * cs - v[2 * j + 1] * sn;
+        hi[j] = v[2 * j + 1] * cs + v[2 * j] * sn;
+      }
+      store4(out + first, lo[0], lo[1], lo[2], lo[3]);
+      store4(out + half + first, hi[0], hi[1], hi[2], hi[3]);
+    } else {
+      store8(out + c, v);
+    }
+  }
+}
+
 }  // namespace tlie
 
 using namespace tlie;
@@ -85,6 +139,25 @@ extern "C" int tlie_rope_cache(const void* qkv, int in_dtype, int nsplit, long l
   if (tokens <= 0 || nq <= 0 || nkv <= 0 || d <= 0 || d > 1024 || page_size <= 0 || nsplit < 1) return kBadArgument;
   if (rot_dim < 0 || rot_dim > d || rot_dim % 2 != 0) return kBadArgument;
   const int heads = nq + 2 * nkv;
+  hipStream_t s = (hipStream_t)stream;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
+                         reinterpret_cast<uintptr_t>(cache)) & 31) == 0;
+  if (nsplit == 1 && (d & 7) == 0 && aligned && (inv_freq == nullptr || (paired && (rot_dim & 7) == 0))) {
+    const int groups = heads * d / 8;
+    const int wide = groups >= 1024 ? 1024 : (groups + 63) / 64 * 64;
+    const size_t wide_lds = static_cast<size_t>(rot_dim) * sizeof(float);
+#define TLIE_WIDE(DC, D, AC, A)                                                                              \
+  if (in_dtype == DC && act_dtype == AC) {                                                                   \
+    hipLaunchKernelGGL((rope_cache_wide_kernel<D, A>), dim3(tokens), dim3(wide), wide_lds, s, (const D*)qkv,   \
+                       positions, slot_map, inv_freq, rot_dim, (A*)q_out, (A*)cache, nq, nkv, d, page_size);  \
+    return launch_status();                                                                                  \
+  }
+    TLIE_WIDE(kF32, float, kF32, float)
+    TLIE_WIDE(kF32, float, kBF16, bf16)
+    TLIE_WIDE(kBF16, bf16, kBF16, bf16)
+#undef TLIE_WIDE
+    return kBadArgument;
+  }
   int heads_per_block = 256 / d;
   if (heads_per_block < 1) heads_per_block = 1;
   if (heads_per_block > heads) heads_per_block = heads;
@@ -92,7 +165,6 @@ extern "C" int tlie_rope_cache(const void* qkv, int in_dtype, int nsplit, long l
   const dim3 grid(tokens, (heads + heads_per_block - 1) / heads_per_block);
   if (grid.y > 65535) return kBadArgument;
   const size_t lds = (static_cast<size_t>(rot_dim) + threads) * sizeof(float);
-  hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(DC, D, AC, A)                                                                              \
   if (in_dtype == DC && act_dtype == AC) {                                                                   \
     hipLaunchKernelGGL((rope_cache_kernel<D, A>), grid, dim3(threads), lds, s, (const D*)qkv, nsplit,         \
