@@ -477,8 +477,12 @@ def test_gemm_rows(shape):
     want = plain_linear(x.double(), w.double(), b.double())
     got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV)).dense()
     assert got.dtype == torch.float32 and rel_err(got, want) < 5e-6
-    for waves in (4, 8, 16):
-        for rows_per_block in (8, 16):
+    for waves in (2, 4, 8, 16):
+        for rows_per_block in (8, 16, 32):
+            if rows_per_block == 32 and waves == 16:
+                with pytest.raises(ops.EngineError):
+                    ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), waves=waves, rows_per_block=rows_per_block)
+                continue
             got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), waves=waves, rows_per_block=rows_per_block).dense()
             assert rel_err(got, want) < 5e-6, (waves, rows_per_block)
     # the norm before the product, folded in: the product runs on residual * g, its rows are scaled
@@ -498,8 +502,8 @@ def test_gemm_rows(shape):
     if n % 2 == 0:
         # rows of W alternate gate and up
         full = plain_linear(x.double(), w.double())
-        for rows_per_block in (8, 16):
-            act = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "silu", rows_per_block=rows_per_block)
+        for rows_per_block, waves in ((8, None), (16, None), (32, 4), (32, 2), (16, 2)):
+            act = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "silu", rows_per_block=rows_per_block, waves=waves)
             assert act.shape == (m, n // 2) and rel_err(act, plain_silu_mul(full[:, 0::2], full[:, 1::2])) < TOL["bfloat16"]
         # the same layout through the kernel that adds up partial sums
         parts = ops.gemm_skinny(x.to(DEV), w.to(DEV), None, split_len=64)
@@ -507,14 +511,19 @@ def test_gemm_rows(shape):
     # added into the residual, with the next norm's inputs
     target = torch.randn(m, n)
     next_g = (1 + 0.2 * torch.randn(n)).bfloat16()
-    for next_weight, rows_per_block in ((next_g, 16), (next_g.float(), 8)):
+    for next_weight, rows_per_block in ((next_g, 16), (next_g.float(), 8), (next_g, 32)):
         res_dev = target.clone().to(DEV)
         updated = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), "residual", residual=res_dev,
-                                next_norm=(next_weight.to(DEV), 1e-6), rows_per_block=rows_per_block)
+                                next_norm=(next_weight.to(DEV), 1e-6), rows_per_block=rows_per_block,
+                                waves=2 if rows_per_block == 32 else None)
         want_res = target.double() + plain_linear(x.double(), w.double(), b.double())
         assert rel_err(res_dev, want_res) < 5e-6
         assert rel_err(updated.normed.xg, want_res * next_g.double()) < TOL["bfloat16"]
-        assert rel_err(updated.normed.ssq[:, :m], partial_sums_of_squares(res_dev.cpu(), rows_per_block)[:, :m]) < 1e-5
+        columns = min(rows_per_block, 16)                  # a block of 32 rows leaves its two strips' sums apart
+        want_ssq = partial_sums_of_squares(res_dev.cpu(), columns)[:, :m]
+        assert updated.normed.ssq.shape[0] >= want_ssq.shape[0]
+        assert rel_err(updated.normed.ssq[:want_ssq.shape[0], :m], want_ssq) < 1e-5
+        assert updated.normed.ssq[want_ssq.shape[0]:, :m].abs().max().item() == 0 if updated.normed.ssq.shape[0] > want_ssq.shape[0] else True
         assert updated.normed.eps == 1e-6
     res_dev = target.clone().to(DEV)
     plain_update = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "residual", residual=res_dev)

@@ -72,34 +72,89 @@ struct RowsArgs {
   uint16_t* cache;            // [pages, 2, nkv, page_size * d]: keys [row][dim], values [dim][row]
 };
 
-// WAVES: 4, 8 or 16 waves share K (more waves for a long K or few strips, fewer when the strips
-// alone fill the chip: every wave costs a dispatch).
-template <int EPILOGUE, int WAVES>
+// WAVES: 2, 4, 8 or 16 waves share K (more waves for a long K or few strips, fewer when the strips
+// alone fill the chip: every wave costs a dispatch).  STRIPS: MFMA strips of 16 rows of W a
+// workgroup (2 when W has rows in plenty: each wave's part of x then serves twice the weights).
+template <int EPILOGUE, int WAVES, int STRIPS>
 __global__ void __launch_bounds__(WAVES * 64)
 gemm_rows_kernel(const RowsArgs a) {
-  __shared__ float partial[WAVES][64][4];           // each wave's 16 x 16 sums
+  __shared__ float partial[STRIPS][WAVES][64][4];   // each wave's 16 x 16 sums per strip
   __shared__ float scale_part[WAVES * 4][16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int block_row = blockIdx.x * a.rows_per_block;
-  const bool row_live = col < a.rows_per_block && block_row + col < a.N;      // with 8 rows a block, half the strip is idle
+  const int strip_rows = STRIPS == 1 ? a.rows_per_block : 16;                 // with 8 rows a block, half the strip is idle
   const int k_begin = wave * a.k_per_wave, k_end = min(a.K, k_begin + a.k_per_wave);
-  const uint16_t* w_row = a.w + static_cast<size_t>(min(block_row + col, a.N - 1)) * a.K;
+  bool row_live[STRIPS];
+  const uint16_t* w_row[STRIPS];
+#pragma unroll
+  for (int st = 0; st < STRIPS; ++st) {
+    row_live[st] = col < strip_rows && block_row + st * 16 + col < a.N;
+    w_row[st] = a.w + static_cast<size_t>(min(block_row + st * 16 + col, a.N - 1)) * a.K;
+  }
   const uint16_t* x_row = a.x + static_cast<size_t>(min(col, a.M - 1)) * a.K;
   const bool token_live = col < a.M;
 
-  floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int k0 = k_begin; k0 < k_end; k0 += 512) {
-    // 512 k of W at once (16 loads of 16 bytes per lane in flight: the weights come from HBM and a
-    // wave has nothing else to do meanwhile); x, which comes from the caches, in two halves
-    RowPack wa[8][2];
+  // the norm's partial sums of squares are asked for before the weights, and added up after the
+  // products: their way from the L2 is hidden behind the weights' way from memory
+  // (the (wave, group) pairs share the strips of the previous product; token = col)
+  constexpr int kScaleLoads = 4;
+  float scale_value[kScaleLoads];
+  const int part = wave * 4 + grp;
+  if (a.ssq_in != nullptr) {
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
-      const int k = k0 + s * 64 + grp * 16;
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-        wa[s][h].u = row_live && k + h * 8 < k_end ? *reinterpret_cast<const uint4*>(w_row + k + h * 8) : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < kScaleLoads; ++i) {
+      const int s = part + i * WAVES * 4;
+      scale_value[i] = s < a.strips_in ? a.ssq_in[s * 16 + col] : 0.f;
     }
+  }
+
+  // What the epilogue needs besides the sums is asked for now as well, for the same reason: each
+  // thread knows its outputs (token = t / 16, row = t % 16 of a strip; see below) from the start.
+  constexpr int kTurns = (256 + WAVES * 64 - 1) / (WAVES * 64);     // outputs of a strip per thread
+  float pre_bias[STRIPS][kTurns], pre_old[STRIPS][kTurns], pre_g[STRIPS][kTurns];
+  float pre_sine[STRIPS][kTurns], pre_cosine[STRIPS][kTurns];
+  int pre_slot[STRIPS][kTurns];
+#pragma unroll
+  for (int st = 0; st < STRIPS; ++st)
+#pragma unroll
+    for (int turn = 0; turn < kTurns; ++turn) {
+      const int t = threadIdx.x + turn * WAVES * 64;
+      const int token = t >> 4, nn = t & 15, n = block_row + st * 16 + nn;
+      const bool live = t < 256 && token < a.M && nn < strip_rows && n < a.N;
+      pre_bias[st][turn] = live && a.bias != nullptr ? bf16_bits_to_float(a.bias[n]) : 0.f;
+      pre_old[st][turn] = pre_g[st][turn] = pre_sine[st][turn] = 0.f;
+      pre_cosine[st][turn] = 1.f;
+      pre_slot[st][turn] = -1;
+      if (EPILOGUE == kEpilogueResidual && live) {
+        pre_old[st][turn] = a.residual[static_cast<size_t>(token) * a.N + n];
+        if (a.xg != nullptr) pre_g[st][turn] = a.next_weight != nullptr ? bf16_bits_to_float(a.next_weight[n]) : a.next_weight_f32[n];
+      }
+      if (EPILOGUE == kEpilogueRope && live) {
+        const int head = n / a.d, p = n % a.d;
+        if (a.inv_freq != nullptr && head < a.nq + a.nkv && p < a.rot_dim)
+          sincosf(static_cast<float>(a.positions[token]) * a.inv_freq[p >> 1], &pre_sine[st][turn], &pre_cosine[st][turn]);
+        if (head >= a.nq) pre_slot[st][turn] = a.slot_map[token];
+      }
+    }
+
+  floatx4 acc[STRIPS];
+#pragma unroll
+  for (int st = 0; st < STRIPS; ++st) acc[st] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = k_begin; k0 < k_end; k0 += 512) {
+    // 512 k of W at once (16 loads of 16 bytes per lane and strip in flight: the weights come from
+    // HBM and a wave has nothing else to do meanwhile); x, which comes from the caches, in two halves
+    RowPack wa[STRIPS][8][2];
+#pragma unroll
+    for (int st = 0; st < STRIPS; ++st)
+#pragma unroll
+      for (int s = 0; s < 8; ++s) {
+        const int k = k0 + s * 64 + grp * 16;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          wa[st][s][h].u = row_live[st] && k + h * 8 < k_end ? *reinterpret_cast<const uint4*>(w_row[st] + k + h * 8)
+                                                             : make_uint4(0, 0, 0, 0);
+      }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       if (k0 + half * 256 >= k_end) break;
@@ -113,104 +168,111 @@ gemm_rows_kernel(const RowsArgs a) {
                                                        : make_uint4(0, 0, 0, 0);
       }
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[half * 4 + s][0].v, xb[s][0].v, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[half * 4 + s][1].v, xb[s][1].v, acc, 0, 0, 0);
-      }
+      for (int st = 0; st < STRIPS; ++st)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[st][half * 4 + s][0].v, xb[s][0].v, acc[st], 0, 0, 0);
+          acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[st][half * 4 + s][1].v, xb[s][1].v, acc[st], 0, 0, 0);
+        }
     }
   }
-  // acc[j] = sum over this wave's k of W[block_row + grp*4 + j][k] * x[col][k]
+  // acc[st][j] = sum over this wave's k of W[block_row + st*16 + grp*4 + j][k] * x[col][k]
 #pragma unroll
-  for (int j = 0; j < 4; ++j) partial[wave][lane][j] = acc[j];
+  for (int st = 0; st < STRIPS; ++st)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) partial[st][wave][lane][j] = acc[st][j];
   if (a.ssq_in != nullptr) {
-    // the (wave, group) pairs share the strips of the previous product; token = col
-    const int part = wave * 4 + grp;
     float sum = 0.f;
-    for (int s = part; s < a.strips_in; s += WAVES * 4) sum += a.ssq_in[s * 16 + col];
+#pragma unroll
+    for (int i = 0; i < kScaleLoads; ++i) sum += scale_value[i];
+    for (int s = part + kScaleLoads * WAVES * 4; s < a.strips_in; s += WAVES * 4) sum += a.ssq_in[s * 16 + col];
     scale_part[part][col] = sum;
   }
   __syncthreads();
 
-  // one thread per output of the strip: token = t / 16, row = t % 16, so a token's outputs sit in
-  // 16 consecutive lanes
-  const int t = threadIdx.x;
-  if (t >= 256) return;       // (with 4 waves every thread has an output)
-  const int token = t >> 4, nn = t & 15, n = block_row + nn;
-  const int from_lane = (nn >> 2) * 16 + token, from_j = nn & 3;    // where the MFMA left this output
-  float value = 0.f;
+  // one thread per output of a strip: token = t / 16, row = t % 16, so a token's outputs sit in
+  // 16 consecutive lanes; the 256 outputs of each strip go round the workgroup's threads (whole
+  // waves at a time: 256 is a multiple of 64)
 #pragma unroll
-  for (int w = 0; w < WAVES; ++w) value += partial[w][from_lane][from_j];
-  if (a.ssq_in != nullptr) {
-    float ssq = 0.f;
+  for (int st = 0; st < STRIPS; ++st)
 #pragma unroll
-    for (int part = 0; part < WAVES * 4; ++part) ssq += scale_part[part][token];
-    value *= rsqrtf(ssq * a.inv_width + a.eps);
-  }
-  const bool live = token < a.M && nn < a.rows_per_block && n < a.N;
-  if (live && a.bias != nullptr) value += bf16_bits_to_float(a.bias[n]);
+    for (int turn = 0; turn < kTurns; ++turn) {
+      const int t = threadIdx.x + turn * WAVES * 64;
+      if (t >= 256) break;                                   // the same for a whole wave
+      const int token = t >> 4, nn = t & 15, n = block_row + st * 16 + nn;
+      const int from_lane = (nn >> 2) * 16 + token, from_j = nn & 3;    // where the MFMA left this output
+      float value = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) value += partial[st][w][from_lane][from_j];
+      if (a.ssq_in != nullptr) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int p = 0; p < WAVES * 4; ++p) ssq += scale_part[p][token];
+        value *= rsqrtf(ssq * a.inv_width + a.eps);
+      }
+      const bool live = token < a.M && nn < strip_rows && n < a.N;
+      value += pre_bias[st][turn];
 
-  if (EPILOGUE == kEpilogueStore) {
-    if (live) a.y[static_cast<size_t>(token) * a.N + n] = value;
-  } else if (EPILOGUE == kEpilogueSilu) {
-    const float up = __shfl_down(value, 1, 64);          // the odd row next to this even one
-    if (live && (nn & 1) == 0) {
-      const float gated = (value / (1.f + expf(-value))) * up;
-      a.act[static_cast<size_t>(token) * (a.N / 2) + (n >> 1)] = __bfloat16_as_ushort(__float2bfloat16(gated));
-    }
-  } else if (EPILOGUE == kEpilogueRope) {
-    const float other = __shfl_xor(value, 1, 64);        // the pair's other element, when this one is rotated
-    if (live) {
-      const int head = n / a.d, p = n % a.d;
-      float result = value;
-      int e = p;
-      if (a.inv_freq != nullptr && head < a.nq + a.nkv && p < a.rot_dim) {
-        const int i = p >> 1, half = a.rot_dim >> 1;
-        float sine, cosine;
-        sincosf(static_cast<float>(a.positions[token]) * a.inv_freq[i], &sine, &cosine);
-        if (p & 1) {
-          e = i + half;
-          result = value * cosine + other * sine;        // second' = second cos + first sin
-        } else {
-          e = i;
-          result = value * cosine - other * sine;        // first' = first cos - second sin
+      if (EPILOGUE == kEpilogueStore) {
+        if (live) a.y[static_cast<size_t>(token) * a.N + n] = value;
+      } else if (EPILOGUE == kEpilogueSilu) {
+        const float up = __shfl_down(value, 1, 64);          // the odd row next to this even one
+        if (live && (nn & 1) == 0) {
+          const float gated = (value / (1.f + expf(-value))) * up;
+          a.act[static_cast<size_t>(token) * (a.N / 2) + (n >> 1)] = __bfloat16_as_ushort(__float2bfloat16(gated));
         }
-      }
-      const uint16_t bits = __bfloat16_as_ushort(__float2bfloat16(result));
-      if (head < a.nq) {
-        a.q_out[(static_cast<size_t>(token) * a.nq + head) * a.d + e] = bits;
+      } else if (EPILOGUE == kEpilogueRope) {
+        const float other = __shfl_xor(value, 1, 64);        // the pair's other element, when this one is rotated
+        if (live) {
+          const int head = n / a.d, p = n % a.d;
+          float result = value;
+          int e = p;
+          if (a.inv_freq != nullptr && head < a.nq + a.nkv && p < a.rot_dim) {
+            const int i = p >> 1, half = a.rot_dim >> 1;
+            const float sine = pre_sine[st][turn], cosine = pre_cosine[st][turn];
+            if (p & 1) {
+              e = i + half;
+              result = value * cosine + other * sine;        // second' = second cos + first sin
+            } else {
+              e = i;
+              result = value * cosine - other * sine;        // first' = first cos - second sin
+            }
+          }
+          const uint16_t bits = __bfloat16_as_ushort(__float2bfloat16(result));
+          if (head < a.nq) {
+            a.q_out[(static_cast<size_t>(token) * a.nq + head) * a.d + e] = bits;
+          } else {
+            const int slot = pre_slot[st][turn];
+            if (slot >= 0) {
+              const size_t head_stride = static_cast<size_t>(a.page_size) * a.d;
+              uint16_t* page = a.cache + static_cast<size_t>(slot / a.page_size) * 2 * a.nkv * head_stride;
+              const int row = slot % a.page_size;
+              if (head < a.nq + a.nkv)
+                page[(head - a.nq) * head_stride + static_cast<size_t>(row) * a.d + e] = bits;
+              else
+                page[(head - a.nq) * head_stride + static_cast<size_t>(e) * a.page_size + row] = bits;
+            }
+          }
+        }
       } else {
-        const int slot = a.slot_map[token];
-        if (slot >= 0) {
-          const size_t head_stride = static_cast<size_t>(a.page_size) * a.d;
-          uint16_t* page = a.cache + static_cast<size_t>(slot / a.page_size) * 2 * a.nkv * head_stride;
-          const int row = slot % a.page_size;
-          if (head < a.nq + a.nkv)
-            page[(head - a.nq) * head_stride + static_cast<size_t>(row) * a.d + e] = bits;
-          else
-            page[(head - a.nq) * head_stride + static_cast<size_t>(e) * a.page_size + row] = bits;
+        float updated = 0.f;
+        if (live) {
+          updated = pre_old[st][turn] + value;
+          a.residual[static_cast<size_t>(token) * a.N + n] = updated;
+          if (a.xg != nullptr)
+            a.xg[static_cast<size_t>(token) * a.N + n] = __bfloat16_as_ushort(__float2bfloat16(updated * pre_g[st][turn]));
+        }
+        if (a.ssq_out != nullptr) {
+          float square = updated * updated;
+          square += __shfl_xor(square, 1, 64);
+          square += __shfl_xor(square, 2, 64);
+          square += __shfl_xor(square, 4, 64);
+          square += __shfl_xor(square, 8, 64);
+          // one row of partial sums per strip of each block of W's rows
+          if (nn == 0) a.ssq_out[(blockIdx.x * STRIPS + st) * 16 + token] = square;
         }
       }
     }
-  } else {
-    float updated = 0.f;
-    if (live) {
-      float* place = a.residual + static_cast<size_t>(token) * a.N + n;
-      updated = *place + value;
-      *place = updated;
-      if (a.xg != nullptr) {
-        const float g = a.next_weight != nullptr ? bf16_bits_to_float(a.next_weight[n]) : a.next_weight_f32[n];
-        a.xg[static_cast<size_t>(token) * a.N + n] = __bfloat16_as_ushort(__float2bfloat16(updated * g));
-      }
-    }
-    if (a.ssq_out != nullptr) {
-      float square = updated * updated;
-      square += __shfl_xor(square, 1, 64);
-      square += __shfl_xor(square, 2, 64);
-      square += __shfl_xor(square, 4, 64);
-      square += __shfl_xor(square, 8, 64);
-      if (nn == 0) a.ssq_out[blockIdx.x * 16 + token] = square;      // one row of partial sums per block of W's rows
-    }
-  }
 }
 
 // residual[t, :] = table[token[t], :] as float; and for the first norm, as the residual epilogue
@@ -246,9 +308,9 @@ using namespace tlie;
 // ssq_in [strips_in, 16] or null (then no row scale); width: the normed input's width.
 // epilogue 0: y float [M, N].  1: act bfloat16 [M, N / 2], N even, W's rows alternating gate, up.
 // 2: residual float [M, N] += y; if xg is given, next_weight [N] (bfloat16 if next_weight_dtype is 1,
-// else float) and xg bfloat16 [M, N]; if ssq_out is given, float [ceil(N / rows_per_block), 16] (all of it is
-// written).
-// waves: 4, 8 or 16, how many waves of a workgroup share K.  rows_per_block: 16 or 8.
+// else float) and xg bfloat16 [M, N]; if ssq_out is given, float [ceil(N / rows_per_block) * max(1, rows_per_block / 16), 16]
+// (all of it is written).
+// waves: 2, 4, 8 or 16, how many waves of a workgroup share K.  rows_per_block: 8, 16, or 32 (32 with at most 8 waves).
 // 3: the rotation and cache write of rope_cache.hip on W's rows in paired order (see above): positions, slot_map [M],
 // inv_freq [rot_dim / 2] or null, q_out bfloat16 [M, nq * d], cache bfloat16 [pages, 2, nkv, page_size * d];
 // N = (nq + 2 nkv) * d.
@@ -258,8 +320,8 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
                               const int* positions, const int* slot_map, const float* inv_freq, int rot_dim, int nq,
                               int nkv, int d, int page_size, void* q_out, void* cache, int waves, int rows_per_block,
                               void* stream) {
-  if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K & 7) != 0 || (waves != 4 && waves != 8 && waves != 16)) return kBadArgument;
-  if (rows_per_block != 16 && rows_per_block != 8) return kBadArgument;
+  if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K & 7) != 0 || (waves != 2 && waves != 4 && waves != 8 && waves != 16)) return kBadArgument;
+  if (rows_per_block != 16 && rows_per_block != 8 && !(rows_per_block == 32 && waves <= 8)) return kBadArgument;
   if (ssq_in != nullptr && (strips_in <= 0 || width <= 0)) return kBadArgument;
   if (epilogue == kEpilogueStore && y == nullptr) return kBadArgument;
   if (epilogue == kEpilogueSilu && (act == nullptr || (N & 1) != 0)) return kBadArgument;
@@ -283,12 +345,20 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
   hipStream_t s = (hipStream_t)stream;
 #define TLIE_CASE(E)                                                                                  \
   if (epilogue == E) {                                                                                \
-    if (waves == 16)                                                                                  \
-      hipLaunchKernelGGL((gemm_rows_kernel<E, 16>), grid, dim3(1024), 0, s, a);                        \
+    if (rows_per_block == 32 && waves == 8)                                                           \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 8, 2>), grid, dim3(512), 0, s, a);                       \
+    else if (rows_per_block == 32 && waves == 4)                                                      \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 4, 2>), grid, dim3(256), 0, s, a);                       \
+    else if (rows_per_block == 32)                                                                    \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 2, 2>), grid, dim3(128), 0, s, a);                       \
+    else if (waves == 16)                                                                             \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 16, 1>), grid, dim3(1024), 0, s, a);                     \
     else if (waves == 8)                                                                              \
-      hipLaunchKernelGGL((gemm_rows_kernel<E, 8>), grid, dim3(512), 0, s, a);                          \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 8, 1>), grid, dim3(512), 0, s, a);                       \
+    else if (waves == 4)                                                                              \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 4, 1>), grid, dim3(256), 0, s, a);                       \
     else                                                                                              \
-      hipLaunchKernelGGL((gemm_rows_kernel<E, 4>), grid, dim3(256), 0, s, a);                          \
+      hipLaunchKernelGGL((gemm_rows_kernel<E, 2, 1>), grid, dim3(128), 0, s, a);                       \
     return launch_status();                                                                           \
   }
   TLIE_CASE(kEpilogueStore)

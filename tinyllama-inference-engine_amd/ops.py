@@ -456,12 +456,16 @@ def gemm_rows_takes(rows: int, weight: torch.Tensor, dtype: torch.dtype) -> bool
 
 
 def gemm_rows_shape(out_features: int, in_features: int) -> tuple[int, int]:
-    """(waves that share K, rows of W per workgroup).  A workgroup per 16 rows; per 8 when that
-    would leave CUs without one (the chip has 256).  Measured on the TinyLlama shapes: 4 waves
-    when the strips alone fill the chip several times over, 16 for a long K, else 8."""
-    rows_per_block = 16 if (out_features + 15) // 16 >= 256 else 8
-    blocks = (out_features + rows_per_block - 1) // rows_per_block
-    waves = 16 if in_features > 4096 else (4 if blocks >= 2048 else 8)
+    """(waves that share K, rows of W per workgroup), measured inside whole decode steps on the
+    TinyLlama shapes: about four thousand waves in all, 4 to 16 a workgroup (11264 rows: 4 waves a
+    strip of 16, 1.15 ms a step against 1.25 with 8; 2560 rows: 16 waves, against 8 another 0.03 ms
+    less); strips of 8 rows where 16 waves on strips of 16 are still too few and K is long
+    (2048 rows, K = 5632).  Two strips a workgroup and 2 waves gained nothing at these sizes."""
+    strips = (out_features + 15) // 16
+    waves = 4
+    while waves < 16 and strips * waves * 2 <= 4096 and in_features >= waves * 2 * 64:
+        waves *= 2
+    rows_per_block = 8 if (waves == 16 and strips * 16 < 3072 and in_features > 4096) else 16
     return waves, rows_per_block
 
 
@@ -534,7 +538,8 @@ def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str 
                 raise invalid_shape("gemm_rows: the next norm's weight needs one entry per output")
             next_code = dtype_code(next_weight.dtype)
             xg = torch.empty((rows, out_features), dtype=torch.bfloat16, device=device)
-            ssq_out = torch.empty(((out_features + rows_per_block - 1) // rows_per_block, 16), dtype=torch.float32, device=device)
+            parts = (out_features + rows_per_block - 1) // rows_per_block * max(1, rows_per_block // 16)
+            ssq_out = torch.empty((parts, 16), dtype=torch.float32, device=device)
     elif epilogue == "rope":
         code = 3
         if rope is None:
