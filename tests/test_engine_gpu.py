@@ -232,6 +232,15 @@ def test_recorded_decode_steps_replay_like_eager_ones(setups, name, dtype):
             for replay in (a, b):
                 replay.engine.finish("g1")
             live.remove("g1")
+        if turn == 19:
+            # a request ends and one of the same name, shorter, takes the same row of the recorded step:
+            # nothing of the first one's block table may serve the second
+            for replay in (a, b):
+                replay.engine.finish("late")
+                for key in [key for key in replay.rows if key[0] == "late"]:
+                    replay.rows[("late before", key[1])] = replay.rows.pop(key)
+                replay.step([("late", follow["g2"][:3], [2])])
+            follow["late"] = request_tokens(name, 91, 40)
         items = [(request, [follow[request][turn]], [0]) for request in live]
         a.step(items)
         b.step(items)

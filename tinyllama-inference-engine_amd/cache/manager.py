@@ -52,6 +52,7 @@ class RequestPages:
     slot: int
     length: int = 0                                        # positions committed so far
     pages: list[list[int]] = field(default_factory=list)   # per group: block index -> page or ABSENT
+    serial: int = 0                                        # which admission this is: no two ever share one
 
 
 class CacheManager:
@@ -72,6 +73,7 @@ class CacheManager:
         self._requests: dict[Hashable, RequestPages] = {}
         self._free_slots = list(range(max_requests - 1, -1, -1))   # popped from the end: slot 0 first
         self._slot_in_use = bytearray(max_requests)
+        self._admissions = 0
         self.state_areas: list[torch.Tensor] = []
 
         group_of_window: dict[int | None, int] = {}
@@ -116,7 +118,8 @@ class CacheManager:
         self._slot_in_use[slot] = 1
         for area in self.state_areas:
             area[slot].zero_()
-        self._requests[request] = RequestPages(slot=slot, pages=[[] for _ in self.groups])
+        self._admissions += 1
+        self._requests[request] = RequestPages(slot=slot, pages=[[] for _ in self.groups], serial=self._admissions)
         return slot
 
     def is_live(self, request: Hashable) -> bool:
@@ -208,6 +211,11 @@ class CacheManager:
 
     def page_list(self, request: Hashable, group: int) -> list[int]:
         return self._entry(request).pages[group]
+
+    def held(self, request: Hashable) -> RequestPages:
+        """What the request holds (to read, not to change).  Its page lists only ever grow at the
+        end or turn entries ABSENT; `serial` tells one admission of a request name from the next."""
+        return self._entry(request)
 
     def rows(self, request: Hashable, group: int, first: int, count: int) -> list[int]:
         """The cache rows (page * page_size + offset) of positions first .. first + count - 1."""

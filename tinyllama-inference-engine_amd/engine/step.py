@@ -217,26 +217,51 @@ class DecodeGraph:
             few_rows=bucket <= 16 and runner.model.dtype == torch.bfloat16, wants_all_rows=True)
         self.graph = None
         self.logits = None
+        self._rows_filled = bucket                           # rows that may hold a step's values
+        self._known = [[(0, 0)] * bucket for _ in cache.groups]   # per group and row: (admission, blocks written)
 
     def _fill(self, entries: Sequence[StepEntry]) -> None:
+        """The step's arrays in the pinned buffer.  A row's part of a block table is kept from
+        step to step while the same admission of a request stays in the row: its page list only
+        grows, so only the new entries are written.  (Entries of pages that a window has given
+        back since keep the old page number: any page number is good there, the kernels mask
+        those positions.)"""
         cache, host, count = self.runner.cache, self.host, len(entries)
+        page_size, shift = cache.page_size, cache.page_size.bit_length() - 1
+        held = [cache.held(entry.request) for entry in entries]
+        positions = [info.length for info in held]
+        stale = max(self._rows_filled, count)
         for name in ("tokens", "positions", "seq_first_pos", "seq_slot"):
-            host[name][count:] = 0
-        host["seq_len"][count:] = 1
-        for row, entry in enumerate(entries):
-            position = cache.length(entry.request)
-            host["tokens"][row] = int(entry.tokens[0])
-            host["positions"][row] = host["seq_first_pos"][row] = position
-            host["seq_len"][row] = position + 1
-            host["seq_slot"][row] = cache.slot(entry.request)
+            host[name][count:stale] = 0
+        host["seq_len"][count:stale] = 1
+        host["tokens"][:count] = [int(entry.tokens[0]) for entry in entries]
+        host["positions"][:count] = positions
+        host["seq_first_pos"][:count] = positions
+        host["seq_len"][:count] = [position + 1 for position in positions]
+        host["seq_slot"][:count] = [info.slot for info in held]
         for group in range(len(cache.groups)):
-            table, slots = host[f"block_table{group}"], host[f"slot_map{group}"]
-            table[count:] = 0
-            slots[count:] = -1
-            for row, entry in enumerate(entries):
-                pages = cache.page_list(entry.request, group)
-                table[row, :len(pages)] = [page if page != ABSENT else 0 for page in pages]
-                slots[row] = cache.rows(entry.request, group, int(host["positions"][row]), 1)[0]
+            table, slots, known = host[f"block_table{group}"], host[f"slot_map{group}"], self._known[group]
+            table[count:stale] = 0
+            slots[count:stale] = -1
+            for row in range(count, stale):
+                known[row] = (0, 0)
+            rows = []
+            for row, info in enumerate(held):
+                pages = info.pages[group]
+                serial, copied = known[row]
+                if serial != info.serial or copied > len(pages):
+                    table[row] = 0
+                    copied = 0
+                if copied < len(pages):
+                    fresh = pages[copied:]
+                    table[row, copied:len(pages)] = [page if page != ABSENT else 0 for page in fresh] if ABSENT in fresh else fresh
+                    known[row] = (info.serial, len(pages))
+                page = pages[positions[row] >> shift]
+                if page == ABSENT:
+                    raise out_of_bounds(f"position {positions[row]} of request {entries[row].request!r} has no page")
+                rows.append(page * page_size + (positions[row] & (page_size - 1)))
+            slots[:count] = rows
+        self._rows_filled = count
 
     def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         runner = self.runner
