@@ -141,7 +141,7 @@ def main() -> int:
     step_bytes = weight_bytes_per_step(cfg, itemsize) + args.batch * mean_context * kv_bytes_per_token(cfg, itemsize)
     achieved = step_bytes / (elapsed / args.steps)
     record = {
-        "metric": "decode tok/s at batch 8, context 2048 (TinyLlama 1.1B shape)", "value": value, "unit": "tokens/s",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (TinyLlama 1.1B shape)", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",

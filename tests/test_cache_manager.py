@@ -71,6 +71,31 @@ def test_pages_follow_length_and_come_back():
     assert caught.value.code == ErrorCode.OUT_OF_BOUNDS           # past the model's positions
 
 
+def test_a_step_reserves_for_all_its_requests_or_for_none():
+    cache = manager()                                             # 8 pages of 4 positions
+    for name in "abc":
+        cache.admit(name)
+    assert cache.reserve_all([("a", 5), ("b", 9)])                # 2 + 3 pages
+    assert cache.page_list("a", 0) == [0, 1] and cache.page_list("b", 0) == [2, 3, 4]
+    cache.commit("a", 5)
+    cache.commit("b", 9)
+    before = cache.held("a").serial, cache.held("b").serial
+    assert not cache.reserve_all([("a", 3), ("c", 9), ("b", 4)])  # 0 + 3 + 1 pages, 3 are free
+    assert cache.page_list("a", 0) == [0, 1] and cache.page_list("c", 0) == [] and cache.free_pages() == [3]
+    assert cache.reserve_all([("a", 3), ("c", 8), ("b", 4)])      # 0 + 2 + 1
+    assert cache.page_list("c", 0) == [5, 6] and cache.page_list("b", 0) == [2, 3, 4, 7]
+    with pytest.raises(EngineError) as caught:
+        cache.reserve_all([("a", 60)])
+    assert caught.value.code == ErrorCode.OUT_OF_BOUNDS
+    with pytest.raises(EngineError):
+        cache.reserve_all([("a", 0)])
+    cache.check()
+    # an admission's serial tells a request's name from its next use
+    cache.release("a")
+    cache.admit("a")
+    assert cache.held("a").serial not in before and cache.held("b").serial == before[1]
+
+
 def test_request_slots_run_out_and_state_starts_at_zero():
     cache = manager(max_requests=2, state=True)
     assert len(cache.state_areas) == 2 and cache.state_areas[0].shape == (2, 5)

@@ -532,14 +532,15 @@ def test_gemm_rows(shape):
 
 def test_embed_rows_and_refusals():
     from tlie_amd import EngineError, ops
-    table = torch.randn(301, 72).bfloat16().to(DEV)
-    g = (1 + 0.2 * torch.randn(72)).bfloat16().to(DEV)
     tokens = torch.tensor([0, 300, 17, 17, 5], dtype=torch.int32, device=DEV)
-    residual, normed = ops.embed_rows(tokens, table, (g, 1e-5))
-    rows = table.float().cpu()[tokens.long().cpu()]
-    assert torch.equal(residual.cpu(), rows)
-    assert rel_err(normed.xg, rows.double() * g.double().cpu()) < TOL["bfloat16"]
-    assert rel_err(normed.ssq[:, :5], partial_sums_of_squares(rows)[:, :5]) < 1e-5
+    for hidden, dtype in ((72, torch.bfloat16), (70, torch.bfloat16), (2056, torch.bfloat16), (40, torch.float32)):
+        table = torch.randn(301, hidden).to(dtype).to(DEV)       # 70: no multiple of 4, one element a thread
+        g = (1 + 0.2 * torch.randn(hidden)).to(dtype).to(DEV)
+        residual, normed = ops.embed_rows(tokens, table, (g, 1e-5))
+        rows = table.float().cpu()[tokens.long().cpu()]
+        assert torch.equal(residual.cpu(), rows)
+        assert rel_err(normed.xg, rows.double() * g.double().cpu()) < TOL["bfloat16"]
+        assert rel_err(normed.ssq[:, :5], partial_sums_of_squares(rows)[:, :5]) < 1e-5
     with pytest.raises(EngineError):
         ops.gemm_rows(torch.randn(17, 64, device=DEV).bfloat16(), torch.randn(8, 64, device=DEV).bfloat16(), None)
     with pytest.raises(EngineError):

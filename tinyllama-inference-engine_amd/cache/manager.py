@@ -179,6 +179,31 @@ class CacheManager:
         for group_index, group in enumerate(self.groups):
             entry.pages[group_index].extend(group.allocator.alloc(needed[group_index]))
 
+    def reserve_all(self, wanted: list[tuple[Hashable, int]]) -> bool:
+        """`reserve` for every (request, more positions) of a step, or for none of them: False when
+        the free pages do not cover them all.  One pass over the requests (a decode step of many
+        requests spends its host time here)."""
+        groups = range(len(self.groups))
+        needs, totals = [], [0] * len(self.groups)
+        for request, count in wanted:
+            entry = self._entry(request)
+            if count <= 0:
+                raise invalid_argument("a request needs at least one new position in a step")
+            if self.max_positions is not None and entry.length + count > self.max_positions:
+                raise out_of_bounds(f"request {request!r} would reach position {entry.length + count - 1}, "
+                                    f"past the model's {self.max_positions} positions")
+            blocks = (entry.length + count + self.page_size - 1) // self.page_size
+            for group in groups:
+                more = blocks - len(entry.pages[group])
+                if more > 0:
+                    needs.append((entry, group, more))
+                    totals[group] += more
+        if any(total > group.allocator.num_free for total, group in zip(totals, self.groups)):
+            return False
+        for entry, group, more in needs:
+            entry.pages[group].extend(self.groups[group].allocator.alloc(more))
+        return True
+
     def commit(self, request: Hashable, count: int) -> None:
         """The step that wrote `count` more positions is enqueued: the request is that much
         longer; a windowed group gives back pages that no later token can see."""

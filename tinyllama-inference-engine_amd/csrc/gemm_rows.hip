@@ -300,6 +300,29 @@ __global__ void embed_rows_kernel(const int* __restrict__ tokens, const W* __res
   }
 }
 
+// The same with four elements a thread and blocks side by side over the row (hidden % 4 == 0):
+// grid (tokens, ceil(hidden / (4 * blockDim.x))).
+template <typename W, typename G>
+__global__ void embed_rows_wide_kernel(const int* __restrict__ tokens, const W* __restrict__ table,
+                                       float* __restrict__ residual, const G* __restrict__ next_weight,
+                                       uint16_t* __restrict__ xg, float* __restrict__ ssq_out, int hidden) {
+  const int t = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  const bool live = i < hidden;
+  float v[4] = {0.f, 0.f, 0.f, 0.f}, g[4] = {0.f, 0.f, 0.f, 0.f};
+  if (live) {
+    const W* row = table + static_cast<size_t>(tokens[t]) * hidden + i;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = to_float(row[j]), g[j] = to_float(next_weight[i + j]);   // adjacent: the compiler joins the loads
+    store4(residual + static_cast<size_t>(t) * hidden + i, v[0], v[1], v[2], v[3]);
+    store4(reinterpret_cast<bf16*>(xg) + static_cast<size_t>(t) * hidden + i, v[0] * g[0], v[1] * g[1], v[2] * g[2], v[3] * g[3]);
+  }
+  float square = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+  square += __shfl_xor(square, 1, 64);
+  square += __shfl_xor(square, 2, 64);
+  if ((threadIdx.x & 3) == 0 && live) ssq_out[(i >> 4) * 16 + t] = square;
+}
+
 }  // namespace tlie
 
 using namespace tlie;
@@ -376,11 +399,18 @@ extern "C" int tlie_embed_rows(const int* tokens, const void* table, int table_d
                                int hidden, void* stream) {
   if (num_tokens <= 0 || num_tokens > 16 || hidden <= 0) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(num_tokens), block(256);
+  const bool wide = (hidden & 3) == 0 &&
+                    ((reinterpret_cast<uintptr_t>(table) | reinterpret_cast<uintptr_t>(residual) |
+                      reinterpret_cast<uintptr_t>(next_weight) | reinterpret_cast<uintptr_t>(xg)) & 15) == 0;
+  const dim3 grid(num_tokens, wide ? (hidden + 1023) / 1024 : 1), block(256);
 #define TLIE_CASE(WC, W, GC, G)                                                                                      \
   if (table_dtype == WC && next_weight_dtype == GC) {                                                                \
-    hipLaunchKernelGGL((embed_rows_kernel<W, G>), grid, block, 0, s, tokens, (const W*)table, residual,               \
-                       (const G*)next_weight, (uint16_t*)xg, ssq_out, hidden);                                       \
+    if (wide)                                                                                                        \
+      hipLaunchKernelGGL((embed_rows_wide_kernel<W, G>), grid, block, 0, s, tokens, (const W*)table, residual,        \
+                         (const G*)next_weight, (uint16_t*)xg, ssq_out, hidden);                                     \
+    else                                                                                                             \
+      hipLaunchKernelGGL((embed_rows_kernel<W, G>), grid, block, 0, s, tokens, (const W*)table, residual,             \
+                         (const G*)next_weight, (uint16_t*)xg, ssq_out, hidden);                                     \
     return launch_status();                                                                                          \
   }
   TLIE_CASE(kBF16, bf16, kBF16, bf16)

@@ -149,10 +149,8 @@ class ModelRunner:
         the entries and of each entry's `want`."""
         self._validate(entries)
         wanted = [(entry.request, len(entry.tokens)) for entry in entries]
-        if not self.cache.can_reserve(wanted):
+        if not self.cache.reserve_all(wanted):
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
-        for request, count in wanted:
-            self.cache.reserve(request, count)
         if self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH and \
                 all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries):
             bucket = DecodeGraph.bucket_of(len(entries))
