@@ -348,3 +348,72 @@ def test_benchmark_layer_sizes_cut_three_ways(tmp_path, dtype):
     engine.finish("p")
     bad = first_bad_row(portions.logits_of("p", range(length)), want, TOLERANCE[dtype])
     assert bad is None, f"portions {sizes}: first wrong position {bad}"
+
+
+def plain_sampled_continuation(setup, prompt, generated, temperature, top_p, seed, tolerance):
+    """Checks a sampled continuation against the plain implementation token by token: token i must be
+    what the plain distribution at that place gives for the uniform number of (seed, i) when the
+    kept tokens are walked in index order, unless that number falls within rounding of a boundary
+    between two tokens.  Returns the number of such near-boundary differences."""
+    from tlie_amd.sampling import uniform01
+    from plain_llama import plain_top_p_distribution
+    near = 0
+    for index, token in enumerate(generated):
+        logits = plain_forward(setup["raw"], setup["weights"], prompt + generated[:index])[-1]
+        distribution = plain_top_p_distribution(logits, temperature, top_p)
+        cumulative = torch.cumsum(distribution, 0)
+        u = uniform01(seed, index)
+        want = min(int(torch.searchsorted(cumulative, torch.tensor(u, dtype=torch.float64)).item()), len(distribution) - 1)
+        if token != want:
+            assert distribution[token] > 0, f"token {index} = {token} is outside the kept set"
+            edge = min(abs(u - cumulative[token].item()), abs(u - (cumulative[token] - distribution[token]).item()))
+            assert edge < tolerance, f"token {index}: drew {token}, the plain walk gives {want} (distance to the boundary {edge:.2e})"
+            near += 1
+    return near
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_seeded_sampling_is_the_same_under_every_cut_and_under_preemption(setups, dtype):
+    """Three requests (prompts of 5, 37 and 64 tokens), temperature 0.8, seeded: together with
+    prompts cut into portions of 16 beside decoded tokens; each alone and whole; and with so few
+    pages that the scheduler has to preempt and recompute.  In 32-bit all three give the same
+    tokens, which are the plain implementation's draws; bfloat16 is checked against the plain draws
+    up to its first near tie."""
+    from tlie_amd import Engine
+    from tlie_amd.engine import Request, SamplingParams, Scheduler
+    name = "B"
+    setup = setups(name, dtype)
+    prompts = [request_tokens(name, 40 + i, n) for i, n in enumerate((5, 37, 64))]
+    new_tokens, temperature, top_p, seed = 24, 0.8, 0.95, 321
+    together = new_engine(setup, dtype).generate(prompts, max_tokens=new_tokens, temperature=temperature, top_p=top_p,
+                                                 seed=seed, chunk_size=16, max_tokens_per_step=24)
+    alone = []
+    for index, prompt in enumerate(prompts):
+        alone += new_engine(setup, dtype).generate([prompt], max_tokens=new_tokens, temperature=temperature, top_p=top_p,
+                                                   seed=seed + index)
+    # 8 pages of 16 positions: the three requests need 2 + 4 + 6 at their ends, so they cannot all stay
+    tight = Engine(setup["folder"], dtype=dtype, max_tokens=128, page_size=16, max_requests=4)
+    assert tight.cache.num_pages == 8
+    scheduler = Scheduler(tight.cache, max_tokens_per_step=24, max_seqs_per_step=4, chunk_size=16,
+                          max_positions=tight.spec.max_positions, eos_token_id=tight.spec.eos_token_id)
+    requests = [Request(id=("tight", i), prompt=list(prompt),
+                        params=SamplingParams(max_tokens=new_tokens, temperature=temperature, top_p=top_p, seed=seed + i))
+                for i, prompt in enumerate(prompts)]
+    for request in requests:
+        scheduler.add(request)
+    tight.run(scheduler)
+    assert scheduler.stats["preemptions"] > 0, "the pool was meant to be too small for all three"
+    assert tight.cache.free_pages() == [8]
+    squeezed = [request.generated for request in requests]
+    assert all(len(tokens) == new_tokens for tokens in together + alone + squeezed)
+    if dtype == "float32":
+        assert together == alone, "cutting and batching changed a seeded draw"
+        assert squeezed == alone, "preemption and recomputation changed a seeded draw"
+        for index, prompt in enumerate(prompts):
+            assert plain_sampled_continuation(setup, prompt, alone[index], temperature, top_p, seed + index, 1e-4) <= 1
+    else:
+        for index, prompt in enumerate(prompts):
+            for tokens in (together[index], alone[index], squeezed[index]):
+                same = next((i for i, (a, b) in enumerate(zip(tokens, alone[index])) if a != b), new_tokens)
+                # up to where two cuts part ways (a near tie for bfloat16), the draws are the plain ones
+                plain_sampled_continuation(setup, prompt, tokens[:same], temperature, top_p, seed + index, 5e-2)
