@@ -132,6 +132,89 @@ def test_attention_part_whole_and_in_portions(dtype, case):
         assert len(held) <= (case["window"] + 7) // 8 + 1, "pages a window has passed were not given back"
 
 
+def test_rotary_part_table_and_refusals():
+    """The position encoding alone: its table is the plain angles at position 1, for the part of
+    the head that turns; sizes that cannot be paired are refused."""
+    from tlie_amd import EngineError
+    from tlie_amd.config import PartSpec
+    from tlie_amd.parts.rotary import NoPositions, Rotary
+    from plain_llama import plain_rope_angles
+    for head_dim, rot_dim, theta in ((64, 64, 10000.0), (48, 16, 500000.0), (16, 2, 3.5)):
+        part = Rotary(PartSpec("rotary", {"head_dim": head_dim, "theta": theta, "rot_dim": rot_dim}), torch.bfloat16, DEV)
+        inv_freq, turned = part.rotary_table()
+        assert turned == rot_dim and inv_freq.dtype == torch.float32 and inv_freq.shape == (rot_dim // 2,)
+        assert torch.equal(inv_freq.cpu(), plain_rope_angles(torch.tensor([1]), rot_dim, theta)[0])
+    assert Rotary(PartSpec("rotary", {"head_dim": 32, "theta": 1e4}), torch.float32, DEV).rotary_table()[1] == 32
+    assert NoPositions(PartSpec("none"), torch.float32, DEV).rotary_table() is None
+    for bad in ({"head_dim": 32, "theta": 1e4, "rot_dim": 7}, {"head_dim": 32, "theta": 1e4, "rot_dim": 34},
+                {"head_dim": 32, "theta": 0.0}):
+        with pytest.raises(EngineError):
+            Rotary(PartSpec("rotary", bad), torch.float32, DEV)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("tied", [False, True])
+def test_embedding_and_head_parts(dtype, tied):
+    """The two ends alone: rows of the table, unscaled, as a 32-bit residual; logits in 32-bit from
+    the head's own matrix or, tied, from the table."""
+    from tlie_amd.config import PartSpec
+    from tlie_amd.parts.embedding import LMHead, TokenEmbedding
+    spec = PartSpec("token_embedding", {"vocab_size": 301, "hidden_size": 72})
+    head_spec = PartSpec("lm_head", {"vocab_size": 301, "hidden_size": 72, "tied": tied})
+    host, device = part_weights(TokenEmbedding, spec, "", DT[dtype], 4)
+    head_host, head_device = part_weights(LMHead, head_spec, "", DT[dtype], 5)
+    assert [t.optional for t in LMHead.tensor_specs(head_spec)] == [tied]
+    embedding, head = TokenEmbedding(spec, DT[dtype], DEV), LMHead(head_spec, DT[dtype], DEV)
+    embedding.load(device)
+    head.load({**device, **({} if tied else head_device)})
+    tokens = torch.tensor([0, 300, 17, 17, 5, 299], dtype=torch.int32, device=DEV)
+    residual = embedding.forward(tokens)
+    assert residual.dtype == torch.float32
+    assert torch.equal(residual.cpu(), host[TokenEmbedding.NAME].float()[tokens.long().cpu()])
+    x = torch.randn(6, 72).to(DT[dtype])
+    logits = head.forward(x.to(DEV))
+    matrix = host[TokenEmbedding.NAME] if tied else head_host[LMHead.NAME]
+    assert logits.dtype == torch.float32 and logits.shape == (6, 301)
+    assert_close(logits, plain_linear(x.double(), matrix.double()), TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [40, 7])
+def test_pre_norm_block_part(dtype, rows):
+    """The arrangement alone: one block of norm, attention, norm, feed-forward around a 32-bit
+    residual, against the plain block; the block's last product is handed on, not added.  With 7
+    rows a bfloat16 step takes the route on which the products fold the norms and the adds in."""
+    from tlie_amd.cache import CacheManager, RunNeed
+    from tlie_amd.config import LlamaConfig
+    from tlie_amd.engine.step import StepEntry, build_context
+    from tlie_amd.ops import ResidualUpdated, as_product
+    from tlie_amd.parts.block import PreNormBlock
+    from tlie_amd.weights import random_tensors
+    from plain_llama import plain_block
+    raw = dict(model_type="llama", hidden_size=72, intermediate_size=200, num_hidden_layers=1, num_attention_heads=6,
+               num_key_value_heads=2, head_dim=16, max_position_embeddings=64, vocab_size=50, rms_norm_eps=2e-5,
+               rope_theta=777.0, attention_bias=True)
+    layer = LlamaConfig.from_dict(raw).to_spec().layers[0]
+    host = random_tensors(PreNormBlock.tensor_specs(layer), 6, std=0.2, norm_std=0.2, dtype=DT[dtype])
+    block = PreNormBlock(layer, DT[dtype], DEV)
+    block.load({name: tensor.to(DEV) for name, tensor in host.items()})
+    cache = CacheManager([RunNeed(0, block.mixer.cache_need(), block.mixer.state_need())], 16, 8, 2, DT[dtype], DEV)
+    cache.admit("r")
+    cache.reserve("r", rows)
+    ctx = build_context(cache, [StepEntry("r", [0] * rows, [])], DEV, few_rows_dtype=DT[dtype])
+    assert ctx.few_rows == (rows <= 16 and dtype == "bfloat16")
+    x = torch.randn(rows, 72)
+    residual = x.clone().to(DEV)
+    pending = block.forward(residual, None, ctx, cache.bindings[0])
+    if isinstance(pending, ResidualUpdated):
+        got = residual                                       # the feed-forward added its result itself
+    else:
+        got = residual + as_product(pending).dense(torch.float32)
+    want = plain_block(x.double(), torch.arange(rows), {name: tensor.double() for name, tensor in host.items()},
+                       layer.prefix, raw)
+    assert_close(got, want, TOL[dtype])
+
+
 # ---------------------------------------------------------------------------------------------------
 # Parts and an architecture defined by the test.
 
