@@ -1,5 +1,5 @@
 """Each part alone against its plain reference, and the generality of the parts: a mixer with state
-of its own, a position encoding that is no rotation, and an architecture of its own, all defined
+of its own, a feed-forward with routing, a position encoding that is no rotation, and an architecture of its own, all defined
 here and registered without a change to the engine's files; a layer order that names a layer twice
 and lets a run read another run's cache; a windowed attention whose pages come back."""
 import json
@@ -221,7 +221,7 @@ def test_pre_norm_block_part(dtype, rows):
 def register_toys():
     from tlie_amd import ops
     from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run, TensorSpec
-    from tlie_amd.parts import Mixer, PositionEncoding, StateNeed
+    from tlie_amd.parts import FeedForward, Mixer, PositionEncoding, StateNeed
     from tlie_amd.parts.linear import Linear
     from tlie_amd.registry import register
 
@@ -249,6 +249,38 @@ def register_toys():
                 binding.state[slot] = sums[-1]
                 means[begin:end] = sums / (ctx.positions[begin:end].float() + 1.0)[:, None]
             return self.mix(means.to(self.dtype).contiguous())
+
+    @register("feed_forward", "toy_routed")
+    class Routed(FeedForward):
+        """A feed-forward with routing: the router's logits (32-bit) choose one of `experts` small
+        two-matrix networks per token; its result is weighted by the router's softmax probability."""
+
+        @classmethod
+        def tensor_specs(cls, spec, prefix):
+            hidden, inter, experts = spec["hidden_size"], spec["intermediate_size"], spec["experts"]
+            specs = [TensorSpec(prefix + "router.weight", (experts, hidden))]
+            for e in range(experts):
+                specs += [TensorSpec(f"{prefix}experts.{e}.up.weight", (inter, hidden)),
+                          TensorSpec(f"{prefix}experts.{e}.down.weight", (hidden, inter))]
+            return specs
+
+        def load(self, weights, prefix):
+            self.router = Linear(weights[prefix + "router.weight"], None, self.dtype)
+            self.experts = [(Linear(weights[f"{prefix}experts.{e}.up.weight"], None, self.dtype),
+                             Linear(weights[f"{prefix}experts.{e}.down.weight"], None, self.dtype))
+                            for e in range(self.spec["experts"])]
+
+        def forward(self, x, ctx):
+            logits = ops.as_product(self.router(x, out_dtype=torch.float32)).dense(torch.float32)
+            probability, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+            out = torch.zeros((x.shape[0], self.spec["hidden_size"]), dtype=torch.float32, device=x.device)
+            for e, (up, down) in enumerate(self.experts):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel() == 0:
+                    continue
+                hidden = torch.relu(ops.as_product(up(x[rows].contiguous())).dense(torch.float32)).to(self.dtype)
+                out[rows] = ops.as_product(down(hidden)).dense(torch.float32) * probability[rows, None]
+            return out.to(self.dtype)
 
     @register("position_encoding", "toy_scale_by_position")
     class ScaleByPosition(PositionEncoding):
@@ -278,8 +310,9 @@ def register_toys():
                                                "bias": False, "window": None, "position": PartSpec("toy_scale_by_position")})
             mean = PartSpec("toy_running_mean", {"hidden_size": self.hidden_size})
             mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 40, "activation": "silu"})
+            routed = PartSpec("toy_routed", {"hidden_size": self.hidden_size, "intermediate_size": 24, "experts": 3})
             layers = (LayerSpec("model.layers.0.", "pre_norm", attention, mlp, norm, norm),
-                      LayerSpec("model.layers.1.", "pre_norm", mean, mlp, norm, norm))
+                      LayerSpec("model.layers.1.", "pre_norm", mean, routed, norm, norm))
             # layer 0 runs three times: with a cache of its own, again with another cache of its own,
             # and once more reading the first run's cache; the toy mixer's layer runs in between
             runs = (Run(0, 0), Run(1, 1), Run(0, 2), Run(0, 0))
@@ -321,7 +354,12 @@ def plain_toy_forward(raw, w, tokens):
     normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)
     means = torch.cumsum(normed, dim=0) / (positions.double() + 1.0)[:, None]
     x = x + plain_linear(means, w[p + "self_attn.mix.weight"])
-    x = x + mlp(x, p)
+    normed = plain_rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
+    probability, choice = torch.softmax(plain_linear(normed, w[p + "mlp.router.weight"]), dim=-1).max(dim=-1)
+    assert len(set(choice.tolist())) > 1, "the routing test wants tokens on more than one expert"
+    routed = torch.stack([plain_linear(torch.relu(plain_linear(normed[t], w[f"{p}mlp.experts.{int(choice[t])}.up.weight"])),
+                                       w[f"{p}mlp.experts.{int(choice[t])}.down.weight"]) * probability[t] for t in range(count)])
+    x = x + routed
     x = attention_run(x, own_cache=2)
     x = attention_run(x, own_cache=None, read=0)
     return plain_linear(plain_rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
