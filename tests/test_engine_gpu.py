@@ -291,6 +291,9 @@ def test_replay_program_and_command_line(setups, tmp_path):
     result = json.loads(run.stdout)
     assert result["prompt_tokens"] == 9
     assert result["generated_tokens"] == plain_generate_greedy(setup["raw"], setup["weights"], tokens[:9], 6)
+    # the step times that the reference's generate reports (app/cuda_reference.cu:216-224)
+    assert all(result[key] > 0 for key in ("prefill_compute_ms", "prefill_transfer_ms", "decode_compute_ms", "decode_transfer_ms"))
+    assert result["prefill_compute_ms"] + result["decode_compute_ms"] < result["wall_ms"]
     run = subprocess.run(cli + ["logits", setup["folder"], prompt, "--dtype", "float32"], capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr
     assert_close(torch.tensor(json.loads(run.stdout)["logits"]), plain_logits(setup, tokens[:9])[-1], TOLERANCE["float32"], "logits")
@@ -417,3 +420,25 @@ def test_seeded_sampling_is_the_same_under_every_cut_and_under_preemption(setups
                 same = next((i for i, (a, b) in enumerate(zip(tokens, alone[index])) if a != b), new_tokens)
                 # up to where two cuts part ways (a near tie for bfloat16), the draws are the plain ones
                 plain_sampled_continuation(setup, prompt, tokens[:same], temperature, top_p, seed + index, 5e-2)
+
+
+def test_step_timings(setups):
+    """A step that is asked for its times waits for the device and reports compute, transfer and
+    wall time, for a prompt step and for a recorded decode step alike; the logits are the same."""
+    from tlie_amd import StepEntry
+    from tlie_amd.engine import StepTimings
+    setup = setups("A", "bfloat16")
+    timed, plain = new_engine(setup, "bfloat16"), new_engine(setup, "bfloat16")
+    tokens = request_tokens("A", 5, 30)
+    for engine in (timed, plain):
+        engine.admit("t")
+    measured = StepTimings()
+    a = timed.step([StepEntry("t", tokens[:20], [19])], measured)
+    b = plain.step([StepEntry("t", tokens[:20], [19])])
+    assert torch.equal(a, b) and 0 < measured.compute_ms < measured.wall_ms and measured.transfer_ms > 0
+    for position in range(20, 30):
+        measured = StepTimings()
+        a = timed.step([StepEntry("t", [tokens[position]], [0])], measured)
+        b = plain.step([StepEntry("t", [tokens[position]], [0])])
+        assert torch.equal(a, b), position
+        assert 0 < measured.compute_ms < measured.wall_ms and measured.transfer_ms > 0

@@ -68,8 +68,9 @@ def command_generate(args) -> int:
     ids, tokenizer = prompt_ids(args.model_dir, args.prompt)
     engine = _engine(args, len(ids) + max_tokens)
     started = time.perf_counter()
+    timings = {}
     generated = engine.generate([ids], max_tokens=max_tokens, temperature=args.temperature, top_p=args.top_p,
-                                seed=args.seed)[0]
+                                seed=args.seed, timings=timings)[0]
     elapsed = (time.perf_counter() - started) * 1e3
     if len(args.rest) > 1:
         try:
@@ -79,7 +80,7 @@ def command_generate(args) -> int:
             raise EngineError(ErrorCode.IO, "unable to open golden metadata") from None
         if len(generated) > len(expected) or list(expected[:len(generated)]) != generated:
             raise EngineError(ErrorCode.NUMERICAL, "greedy tokens do not match the golden tokens")
-    result = {"prompt_tokens": len(ids), "generated_tokens": generated, "wall_ms": elapsed}
+    result = {"prompt_tokens": len(ids), "generated_tokens": generated, "wall_ms": elapsed, **timings}
     if tokenizer is not None:
         result["text"] = tokenizer.decode(generated)
     print(json.dumps(result))

@@ -21,7 +21,7 @@ from ..registry import config_from_dict
 from ..weights.store import WeightStore
 from ..sampling.sampler import Sampler
 from .scheduler import Request, SamplingParams, Scheduler
-from .step import ModelRunner, StepEntry
+from .step import ModelRunner, StepEntry, StepTimings
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "f32": torch.float32,
            "fp32": torch.float32}
@@ -76,16 +76,19 @@ class Engine:
     def finish(self, request: Hashable) -> None:
         self.cache.release(request)
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        return self.runner.step(entries)
+    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
+        return self.runner.step(entries, timings)
 
     # ---- generation -------------------------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,
                  top_p: float = 1.0, seed: int = 0, stop_on_eos: bool = False, max_tokens_per_step: int = 2048,
-                 max_seqs_per_step: int | None = None, chunk_size: int | None = None) -> list[list[int]]:
+                 max_seqs_per_step: int | None = None, chunk_size: int | None = None,
+                 timings: dict | None = None) -> list[list[int]]:
         """Token ids in, generated token ids out, one list per prompt.  Request i samples with
         seed + i.  All prompts run together under the scheduler (continuous batching, prompts cut
-        into portions under the token budget)."""
+        into portions under the token budget).  `timings`: a dict that receives the sums of the
+        steps' compute and transfer times, apart for steps that bring prompt tokens and steps that
+        only decode (the keys of the reference's `generate`, app/cuda_reference.cu:216-224)."""
         scheduler = Scheduler(self.cache, max_tokens_per_step=max_tokens_per_step,
                               max_seqs_per_step=max_seqs_per_step or self.cache.max_requests, chunk_size=chunk_size,
                               max_positions=self.spec.max_positions, eos_token_id=self.spec.eos_token_id)
@@ -96,19 +99,29 @@ class Engine:
             request = Request(id=("generate", index), prompt=[int(token) for token in prompt], params=params)
             scheduler.add(request)
             requests.append(request)
-        self.run(scheduler)
+        self.run(scheduler, timings)
         return [request.generated for request in requests]
 
-    def run(self, scheduler: Scheduler) -> None:
+    def run(self, scheduler: Scheduler, timings: dict | None = None) -> None:
         """The engine loop: plan a step, run it, sample, record; until nothing is left."""
         sampler = Sampler(self.device)
+        if timings is not None:
+            for key in ("prefill_compute_ms", "prefill_transfer_ms", "decode_compute_ms", "decode_transfer_ms"):
+                timings.setdefault(key, 0.0)
         while scheduler.has_work():
             plan = scheduler.schedule()
             if not plan:
                 raise EngineError(ErrorCode.OUT_OF_MEMORY, "no request can make progress with the pages that are free")
             entries = [StepEntry(item.request.id, item.request.tokens[item.first:item.first + item.count],
                                  [item.count - 1] if item.samples else []) for item in plan]
-            logits = self.step(entries)
+            if timings is None:
+                logits = self.step(entries)
+            else:
+                measured = StepTimings()
+                logits = self.step(entries, measured)
+                phase = "decode" if all(item.count == 1 and item.samples and item.request.generated for item in plan) else "prefill"
+                timings[phase + "_compute_ms"] += measured.compute_ms
+                timings[phase + "_transfer_ms"] += measured.transfer_ms
             sampling = [item for item in plan if item.samples]
             tokens = sampler.sample(logits, [item.request.params for item in sampling],
                                     [len(item.request.generated) for item in sampling])

@@ -28,6 +28,18 @@ class StepEntry:
 
 
 @dataclass
+class StepTimings:
+    """Where a step's time went, in milliseconds, when asked for (the step then waits for the
+    device before it returns).  reference: CudaStepTimings, compute / transfer / wall
+    (include/tlie/cuda/model.hpp:14-18), filled by ForwardBatch (src/cuda/model.cu:512-526).
+    transfer: the step's arrays to the device (logits stay on the device here); compute: the
+    model's kernels; wall: the whole call on the host, with validation and page reservation."""
+    compute_ms: float = 0.0
+    transfer_ms: float = 0.0
+    wall_ms: float = 0.0
+
+
+@dataclass
 class GroupView:
     """One page group as the kernels see it in this step."""
     block_table: torch.Tensor      # int32 [sequences, max_blocks]; absent entries hold page 0 and are never read
@@ -143,23 +155,39 @@ class ModelRunner:
         return build_context(self.cache, entries, self.device, few_rows_dtype=self.model.dtype)
 
     # ---- the step ----------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
         """Runs exactly the tokens the entries bring, as one batch, from the cache that earlier
         steps left.  Returns float32 logits [wanted places, vocab] on the device, in the order of
-        the entries and of each entry's `want`."""
+        the entries and of each entry's `want`.  With `timings` the step is timed with events
+        on its stream and waits for them before it returns."""
+        marks = None
+        if timings is not None:
+            import time
+            started = time.perf_counter()
+            marks = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
         self._validate(entries)
         wanted = [(entry.request, len(entry.tokens)) for entry in entries]
         if not self.cache.reserve_all(wanted):
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
+        if marks:
+            marks[0].record()
         if self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH and \
                 all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries):
             bucket = DecodeGraph.bucket_of(len(entries))
             if bucket not in self._graphs:
                 self._graphs[bucket] = DecodeGraph(self, bucket)
-            logits = self._graphs[bucket].run(entries)
+            logits = self._graphs[bucket].run(entries, marks[1] if marks else None)
         else:
             ctx = self.build_context(entries)
+            if marks:
+                marks[1].record()
             logits = self.model.forward(ctx, self.cache.bindings)
+        if marks:
+            marks[2].record()
+            marks[2].synchronize()
+            timings.transfer_ms = marks[0].elapsed_time(marks[1])
+            timings.compute_ms = marks[1].elapsed_time(marks[2])
+            timings.wall_ms = (time.perf_counter() - started) * 1e3
         for request, count in wanted:
             self.cache.commit(request, count)
         return logits
@@ -261,10 +289,13 @@ class DecodeGraph:
             slots[:count] = rows
         self._rows_filled = count
 
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], transferred=None) -> torch.Tensor:
+        """`transferred`: an event to record once the step's arrays are on their way."""
         runner = self.runner
         self._fill(entries)
         self.device_flat.copy_(self.pinned, non_blocking=True)
+        if transferred is not None:
+            transferred.record()
         if self.graph is None:
             # the first step of this size runs eagerly (its result is used, and it leaves the
             # context's work lists made); the same launches are then recorded for the steps to come
