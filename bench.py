@@ -54,36 +54,29 @@ def prefill_flops(cfg, tokens):
 
 
 def time_decode(engine, torch, batch, context, steps, warmup, vocab):
-    """Prefills `batch` requests, runs warmup + steps decode steps ending at `context` positions;
-    returns seconds for the timed steps."""
-    from tlie_amd import StepEntry
-    from tlie_amd.engine import SamplingParams
-    from tlie_amd.sampling import Sampler
-    sampler = Sampler(engine.device)
-    params = [SamplingParams() for _ in range(batch)]
-    prompt_len = context - steps - warmup
+    """`batch` requests through the engine's own loop (scheduler, recorded decode steps, sampling
+    on the device, tokens read a step behind): prompts first, then warmup + steps decode steps, the
+    last token of each request being the `context`-th of its sequence; returns seconds for the
+    timed steps."""
+    from tlie_amd.engine import Request, SamplingParams, Scheduler
+    prompt_len = context - steps - warmup - 1
     generator = torch.Generator().manual_seed(batch)
-    requests = [("bench", index) for index in range(batch)]
-    tokens = []
+    # the token budget lets all prompts through in one step, so that every request decodes from the same step on
+    scheduler = Scheduler(engine.cache, max_tokens_per_step=batch * prompt_len, max_seqs_per_step=batch,
+                          max_positions=engine.spec.max_positions, eos_token_id=engine.spec.eos_token_id)
+    requests = [Request(id=("bench", index), prompt=torch.randint(0, vocab, (prompt_len,), generator=generator).tolist(),
+                        params=SamplingParams(max_tokens=steps + warmup + 1)) for index in range(batch)]
     for request in requests:
-        prompt = torch.randint(0, vocab, (prompt_len,), generator=generator).tolist()
-        engine.admit(request)
-        logits = engine.step([StepEntry(request, prompt, [prompt_len - 1])])
-        tokens.append(sampler.sample(logits, params[:1], [0])[0])
-
-    def run(count):
-        nonlocal tokens
-        for index in range(count):
-            logits = engine.step([StepEntry(request, [token], [0]) for request, token in zip(requests, tokens)])
-            tokens = sampler.sample(logits, params, [index] * batch)
-    run(warmup)
+        scheduler.add(request)
+    assert engine.run(scheduler, max_steps=1) == 1
+    assert all(len(request.generated) == 1 for request in requests)
+    assert engine.run(scheduler, max_steps=warmup) == warmup
     torch.cuda.synchronize()
     started = time.perf_counter()
-    run(steps)
+    ran = engine.run(scheduler, max_steps=steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
-    for request in requests:
-        engine.finish(request)
+    assert ran == steps and not scheduler.has_work() and all(len(request.generated) == steps + warmup + 1 for request in requests)
     return elapsed
 
 

@@ -204,6 +204,8 @@ def test_greedy_generation_through_the_entry_point(setups, name, dtype):
                 gap = (logits[want[same]] - logits[tokens[same]]).item()
                 assert 0 <= gap <= 2 * TOLERANCE[dtype] * logits.abs().max().item(), f"token {same} differs without a near tie"
     assert engine.cache.free_pages() == [engine.cache.num_pages]
+    # the loop launched decode steps before it had read the tokens of the step before
+    assert engine.stats["steps_ahead"] >= 10 and engine.stats["steps_ahead"] <= engine.stats["steps"]
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
@@ -442,3 +444,26 @@ def test_step_timings(setups):
         b = plain.step([StepEntry("t", [tokens[position]], [0])])
         assert torch.equal(a, b), position
         assert 0 < measured.compute_ms < measured.wall_ms and measured.transfer_ms > 0
+
+
+def test_a_request_that_stops_at_a_token_beside_one_that_does_not(setups):
+    """Stopping at the end-of-sequence token needs the token on the host before the next plan:
+    such a request keeps the loop from running ahead, and ends where the token first appears;
+    the request beside it is not disturbed, and the loop runs ahead again once it is alone."""
+    from tlie_amd.engine import Request, SamplingParams, Scheduler
+    setup = setups("A", "float32")
+    prompt, other_prompt = request_tokens("A", 61, 12), request_tokens("A", 62, 20)
+    free = new_engine(setup, "float32").generate([prompt, other_prompt], max_tokens=14)
+    stop_token = free[0][5]
+    want = free[0][:free[0].index(stop_token) + 1]
+    engine = new_engine(setup, "float32")
+    scheduler = Scheduler(engine.cache, max_positions=engine.spec.max_positions, eos_token_id=stop_token)
+    stopper = Request("s", list(prompt), SamplingParams(max_tokens=14, stop_on_eos=True))
+    other = Request("o", list(other_prompt), SamplingParams(max_tokens=14))
+    scheduler.add(stopper)
+    scheduler.add(other)
+    engine.run(scheduler)
+    assert stopper.generated == want and stopper.finish_reason == "eos"
+    assert other.generated == free[1] and other.finish_reason == "length"
+    assert 0 < engine.stats["steps_ahead"] <= engine.stats["steps"] - len(want)
+    assert engine.cache.free_pages() == [engine.cache.num_pages]

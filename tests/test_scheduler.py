@@ -173,3 +173,94 @@ def test_abort_and_eos():
     scheduler2.add(b)
     drive(cache2, scheduler2)
     assert b.finish_reason == "eos" and len(b.generated) == 1
+
+
+def drive_a_step_behind(cache, scheduler, max_steps=500):
+    """As the engine loop runs when the host is one step behind the device: a step's tokens are
+    written into the requests only after the next step has been planned and 'launched'; plans that
+    need a token earlier (a recomputation after a preemption) get it first.  Returns how many
+    steps were planned without the tokens of the step before."""
+    behind, ahead = None, 0
+
+    def settle():
+        nonlocal behind
+        if behind is not None:
+            scheduler.resolve(*behind)
+            behind = None
+
+    for _ in range(max_steps):
+        if not scheduler.has_work():
+            settle()
+            return ahead
+        plan = scheduler.schedule()
+        assert plan, "no progress"
+        for item in plan:
+            request = item.request
+            if request.pending and item.first + item.count == request.total and item.count != 1:
+                settle()                                   # a recomputed portion reaches the pending token
+        ahead += behind is not None
+        for item in plan:
+            cache.reserve(item.request.id, item.count)
+            cache.commit(item.request.id, item.count)
+        known = behind
+        settle()                                           # "while the step runs"
+        sampled = [fake_token(item.request.token_slice(0, item.first + item.count)) for item in plan if item.samples]
+        assert known is None or all(token >= 0 for item in plan for token in item.request.token_slice(0, item.first + item.count))
+        if scheduler.can_defer(plan):
+            scheduler.update(plan, None)
+            behind = (plan, sampled)
+        else:
+            scheduler.update(plan, sampled)
+        cache.check()
+    raise AssertionError("did not finish")
+
+
+def test_tokens_may_arrive_a_step_late():
+    from tlie_amd.engine.scheduler import PENDING
+    # ample pages: every decode step is planned before the last one's tokens are in
+    cache, scheduler = make(num_pages=32, max_tokens_per_step=8, chunk_size=4)
+    requests = [Request(name, list(range(3 + 2 * i, 9 + 3 * i)), SamplingParams(max_tokens=7 + i)) for i, name in enumerate("abc")]
+    for request in requests:
+        scheduler.add(request)
+    ahead = drive_a_step_behind(cache, scheduler)
+    assert ahead > 10
+    for request in requests:
+        assert request.generated == expected_output(request.prompt, request.params.max_tokens) and request.finish_reason == "length"
+    # few pages: preemptions recompute prompts that end in a token still pending; the output is the same
+    cache, scheduler = make(num_pages=7, max_tokens_per_step=16)
+    requests = [Request(name, [i + 1, i + 2, i + 3, i + 4, i + 5], SamplingParams(max_tokens=12)) for i, name in enumerate("abc")]
+    for request in requests:
+        scheduler.add(request)
+    drive_a_step_behind(cache, scheduler)
+    assert scheduler.stats["preemptions"] > 0
+    for request in requests:
+        assert request.generated == expected_output(request.prompt, 12)
+    # a request that stops at the end-of-sequence token cannot wait for its tokens
+    eos = expected_output([4, 5], 3)[2]
+    cache, scheduler = make(eos_token_id=eos)
+    stopper = Request("s", [4, 5], SamplingParams(max_tokens=50, stop_on_eos=True))
+    other = Request("o", [9, 9, 9], SamplingParams(max_tokens=6))
+    scheduler.add(stopper)
+    scheduler.add(other)
+    drive_a_step_behind(cache, scheduler)
+    assert stopper.finish_reason == "eos" and stopper.generated == expected_output([4, 5], 3)
+    assert other.generated == expected_output([9, 9, 9], 6)
+    # resolve refuses what update did not leave pending
+    cache, scheduler = make()
+    request = Request("r", [1, 2], SamplingParams(max_tokens=3))
+    scheduler.add(request)
+    plan = scheduler.schedule()
+    scheduler.update(plan, None)
+    assert request.generated == [PENDING] and request.pending
+    scheduler.resolve(plan, [55])
+    assert request.generated == [55] and not request.pending
+    with pytest.raises(EngineError):
+        scheduler.resolve(plan, [56])
+
+
+def test_token_slice_is_the_slice_of_prompt_and_generated():
+    request = Request("r", [10, 11, 12, 13], SamplingParams(max_tokens=9), generated=[20, 21, 22])
+    for first in range(7):
+        for count in range(0, 8 - first):
+            assert request.token_slice(first, count) == request.tokens[first:first + count]
+    assert request.total == 7

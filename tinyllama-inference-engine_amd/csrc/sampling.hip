@@ -148,6 +148,21 @@ sample_kernel(const float* __restrict__ logits, int vocab, const float* __restri
 using namespace tlie;
 
 // temperature, top_p, seed, counter: arrays of `rows` entries, or null (greedy for every row).
+// tokens[i] = sampled[source[i]] where source[i] >= 0: a decode step whose tokens are the last step's
+// samples takes them on the device, before the host has read them.
+__global__ void feed_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ source,
+                                   const int* __restrict__ sampled, int count) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count && source[i] >= 0) tokens[i] = sampled[source[i]];
+}
+
+extern "C" int tlie_feed_tokens(int* tokens, const int* source, const int* sampled, int count, void* stream) {
+  if (count <= 0) return kBadArgument;
+  hipLaunchKernelGGL(feed_tokens_kernel, dim3((count + 63) / 64), dim3(64), 0, (hipStream_t)stream, tokens, source,
+                     sampled, count);
+  return launch_status();
+}
+
 extern "C" int tlie_sample(const float* logits, int rows, int vocab, const float* temperature, const float* top_p,
                            const long long* seed, const long long* counter, int* out, void* stream) {
   if (rows <= 0 || vocab <= 0) return kBadArgument;

@@ -68,6 +68,9 @@ class Engine:
         self.cache = CacheManager(self.model.run_needs(), page_size, num_pages, max_requests, self.dtype, self.device,
                                   max_positions=self.spec.max_positions)
         self.runner = ModelRunner(self.model, self.cache, use_graphs=use_graphs)
+        self.sampler = Sampler(self.device, capacity=max(max_requests, 1))
+        self.runner.device_tokens = self.sampler.device_tokens
+        self.stats = {"steps": 0, "steps_ahead": 0}      # steps run by `run`; those whose tokens were read a step later
 
     # ---- the step function and what goes with it --------------------------------------------------
     def admit(self, request: Hashable) -> int:
@@ -102,27 +105,89 @@ class Engine:
         self.run(scheduler, timings)
         return [request.generated for request in requests]
 
-    def run(self, scheduler: Scheduler, timings: dict | None = None) -> None:
-        """The engine loop: plan a step, run it, sample, record; until nothing is left."""
-        sampler = Sampler(self.device)
+    def run(self, scheduler: Scheduler, timings: dict | None = None, max_steps: int | None = None) -> int:
+        """The engine loop: plan a step, run it, sample, record; until nothing is left, or for
+        `max_steps` steps.  Returns the number of steps run.
+
+        The host stays one step behind the device where it can: a decode step's tokens are the
+        last step's samples, which the recorded step takes from the sampler's device buffer, so
+        the step is launched before those tokens have been read; they are read (and written into
+        their requests) while it runs.  What the next plan depends on is known without them,
+        unless a request stops at the end-of-sequence token or the plan has to recompute a
+        preempted request: then the loop waits for the tokens first."""
+        sampler = self.sampler
         if timings is not None:
             for key in ("prefill_compute_ms", "prefill_transfer_ms", "decode_compute_ms", "decode_transfer_ms"):
                 timings.setdefault(key, 0.0)
-        while scheduler.has_work():
-            plan = scheduler.schedule()
-            if not plan:
-                raise EngineError(ErrorCode.OUT_OF_MEMORY, "no request can make progress with the pages that are free")
-            entries = [StepEntry(item.request.id, item.request.tokens[item.first:item.first + item.count],
-                                 [item.count - 1] if item.samples else []) for item in plan]
-            if timings is None:
-                logits = self.step(entries)
+        steps = 0
+        behind = None            # (plan, PendingTokens, {request id: row}) of a step whose tokens the requests still lack
+
+        def settle():
+            nonlocal behind
+            if behind is not None:
+                scheduler.resolve(behind[0], behind[1].read())
+                behind = None
+
+        try:
+            while scheduler.has_work() and (max_steps is None or steps < max_steps):
+                plan = scheduler.schedule()
+                if not plan:
+                    raise EngineError(ErrorCode.OUT_OF_MEMORY, "no request can make progress with the pages that are free")
+                sources = self._device_sources(plan, behind)
+                if sources is None:
+                    settle()
+                    sources = [None] * len(plan)
+                entries = [StepEntry(item.request.id,
+                                     [0] if source is not None else item.request.token_slice(item.first, item.count),
+                                     [item.count - 1] if item.samples else [], source)
+                           for item, source in zip(plan, sources)]
+                if timings is None:
+                    logits = self.step(entries)
+                else:
+                    measured = StepTimings()
+                    logits = self.step(entries, measured)
+                    phase = "decode" if all(item.count == 1 and item.samples and item.request.generated for item in plan) else "prefill"
+                    timings[phase + "_compute_ms"] += measured.compute_ms
+                    timings[phase + "_transfer_ms"] += measured.transfer_ms
+                sampling = [item for item in plan if item.samples]
+                pending = sampler.sample_async(logits, [item.request.params for item in sampling],
+                                               [len(item.request.generated) for item in sampling])
+                settle()                                      # the step before this one, while this one runs
+                steps += 1
+                self.stats["steps"] += 1
+                if scheduler.can_defer(plan) and sampling:
+                    scheduler.update(plan, None)
+                    behind = (plan, pending, {item.request.id: row for row, item in enumerate(sampling)})
+                    self.stats["steps_ahead"] += 1
+                else:
+                    scheduler.update(plan, pending.read())
+        finally:
+            if behind is not None:
+                # also when a step raised: the requests get the tokens that were sampled for them
+                plan, pending, _ = behind
+                behind = None
+                scheduler.resolve(plan, pending.read())
+        return steps
+
+    def _device_sources(self, plan, behind):
+        """For a plan whose step the recording replays: per item the row of the sampler's device
+        tokens that is its token (None: the token is on the host).  None when some token that the
+        plan needs is neither on the host nor a row of the last step's samples, or the step is
+        not replayed."""
+        if behind is None:
+            return [None] * len(plan)
+        rows = behind[2]
+        sources = []
+        for item in plan:
+            request = item.request
+            if not (request.pending and item.first + item.count == request.total):
+                sources.append(None)                          # its tokens are all on the host
+            elif item.count == 1 and request.id in rows:
+                sources.append(rows[request.id])
             else:
-                measured = StepTimings()
-                logits = self.step(entries, measured)
-                phase = "decode" if all(item.count == 1 and item.samples and item.request.generated for item in plan) else "prefill"
-                timings[phase + "_compute_ms"] += measured.compute_ms
-                timings[phase + "_transfer_ms"] += measured.transfer_ms
-            sampling = [item for item in plan if item.samples]
-            tokens = sampler.sample(logits, [item.request.params for item in sampling],
-                                    [len(item.request.generated) for item in sampling])
-            scheduler.update(plan, tokens)
+                return None
+        if any(source is not None for source in sources):
+            probe = [StepEntry(item.request.id, [0] * item.count, [item.count - 1] if item.samples else []) for item in plan]
+            if not self.runner.replays(probe):
+                return None
+        return sources

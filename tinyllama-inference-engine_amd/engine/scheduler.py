@@ -51,6 +51,9 @@ class SamplingParams:
             raise invalid_argument("top_p must be in (0, 1]")
 
 
+PENDING = -1        # in a request's generated tokens: sampled, but not yet read from the device
+
+
 @dataclass
 class Request:
     id: Hashable
@@ -66,6 +69,25 @@ class Request:
     @property
     def tokens(self) -> list[int]:
         return self.prompt + self.generated
+
+    @property
+    def total(self) -> int:
+        """How many tokens the request has: prompt and generated."""
+        return len(self.prompt) + len(self.generated)
+
+    def token_slice(self, first: int, count: int) -> list[int]:
+        """tokens[first : first + count] without joining the two lists."""
+        split = len(self.prompt)
+        if first + count <= split:
+            return self.prompt[first:first + count]
+        if first >= split:
+            return self.generated[first - split:first - split + count]
+        return self.prompt[first:] + self.generated[:first + count - split]
+
+    @property
+    def pending(self) -> bool:
+        """The last generated token has been sampled but is not on the host yet."""
+        return bool(self.generated) and self.generated[-1] == PENDING
 
     @property
     def remaining(self) -> int:
@@ -152,7 +174,7 @@ class Scheduler:
             nonlocal budget
             for group, need in enumerate(self.cache.pages_needed(request.id, count)):
                 planned_pages[group] += need
-            plan.append(Scheduled(request, request.computed, count, request.computed + count == len(request.tokens)))
+            plan.append(Scheduled(request, request.computed, count, request.computed + count == request.total))
             budget -= count
 
         # 1. requests that decode: one token each, from the cursor when they exceed the budget
@@ -228,9 +250,14 @@ class Scheduler:
         self.waiting.appendleft(victim)
 
     # ---- after the step ----------------------------------------------------------------------------
-    def update(self, plan: list[Scheduled], sampled: list[int]) -> list[Request]:
+    def update(self, plan: list[Scheduled], sampled: list[int] | None) -> list[Request]:
         """`sampled` holds one token for each planned item with `samples`, in plan order.
-        Returns the requests that finished."""
+        Returns the requests that finished.
+
+        `sampled` may be None when the tokens are not on the host yet: PENDING stands in their
+        place, and `resolve` writes them later.  Everything a plan depends on is known without
+        them (a request ends by its count of tokens), except the end of a request that stops at
+        the end-of-sequence token: `can_defer` says whether a plan has such a request."""
         done = []
         cursor = 0
         for item in plan:
@@ -238,7 +265,7 @@ class Scheduler:
             request.computed += item.count
             if not item.samples:
                 continue
-            token = int(sampled[cursor])
+            token = PENDING if sampled is None else int(sampled[cursor])
             cursor += 1
             request.generated.append(token)
             if len(request.generated) >= request.params.max_tokens:
@@ -248,6 +275,26 @@ class Scheduler:
                 self._finish(request, "eos")
                 done.append(request)
         return done
+
+    @staticmethod
+    def can_defer(plan: list[Scheduled]) -> bool:
+        """Whether `update` can do without the tokens of this plan's step for now."""
+        return all(not item.request.params.stop_on_eos for item in plan if item.samples)
+
+    @staticmethod
+    def resolve(plan: list[Scheduled], sampled: list[int]) -> None:
+        """The tokens of a plan that `update` took without them.  Item i's token is the one it
+        appended: at index first + count - len(prompt) of the request's generated tokens."""
+        cursor = 0
+        for item in plan:
+            if not item.samples:
+                continue
+            request = item.request
+            index = item.first + item.count - len(request.prompt)
+            if not (0 <= index < len(request.generated)) or request.generated[index] != PENDING:
+                raise invalid_argument(f"request {request.id!r} has no token pending at {index}")
+            request.generated[index] = int(sampled[cursor])
+            cursor += 1
 
     def _finish(self, request: Request, reason: str) -> None:
         if request.state == "running":

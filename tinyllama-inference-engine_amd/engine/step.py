@@ -17,6 +17,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import ABSENT, CacheManager
+from ..ops import feed_tokens as ops_feed_tokens
 from ..errors import invalid_argument, out_of_bounds, out_of_memory
 
 
@@ -25,6 +26,10 @@ class StepEntry:
     request: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = field(default_factory=list)    # places among `tokens` whose logits are asked for
+    # The entry's one token is not on the host yet: it is row `source` of the device tokens that
+    # the last step's sampling left (`ModelRunner.device_tokens`); `tokens` then holds a stand-in.
+    # Only a step of single tokens that is replayed from a recording takes such entries.
+    source: int | None = None
 
 
 @dataclass
@@ -126,6 +131,7 @@ class ModelRunner:
         # kernels are all this engine's own is captured once per batch-size bucket as a HIP graph
         # and replayed.  Parts say whether they may be captured (`graph_safe`).
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
+        self.device_tokens: torch.Tensor | None = None     # int32, where sampling leaves a step's tokens (set by the engine)
         self._graphs: dict[int, "DecodeGraph"] = {}
 
     # ---- checks and context ------------------------------------------------------------------
@@ -139,6 +145,9 @@ class ModelRunner:
             seen.add(entry.request)
             if len(entry.tokens) == 0:
                 raise invalid_argument(f"request {entry.request!r} brings no tokens")
+            if entry.source is not None and (self.device_tokens is None or len(entry.tokens) != 1
+                                             or not 0 <= entry.source < self.device_tokens.shape[0]):
+                raise invalid_argument(f"request {entry.request!r} names a device token that is not there")
             for token in entry.tokens:
                 if not 0 <= int(token) < self.vocab_size:
                     raise out_of_bounds(f"token {token} of request {entry.request!r} is outside the vocabulary of {self.vocab_size}")
@@ -153,6 +162,11 @@ class ModelRunner:
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         return build_context(self.cache, entries, self.device, few_rows_dtype=self.model.dtype)
+
+    def replays(self, entries: Sequence[StepEntry]) -> bool:
+        """Whether the step is one of single tokens, every logit wanted, that a recording serves."""
+        return (self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH
+                and all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries))
 
     # ---- the step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
@@ -171,13 +185,14 @@ class ModelRunner:
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         if marks:
             marks[0].record()
-        if self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH and \
-                all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries):
+        if self.replays(entries):
             bucket = DecodeGraph.bucket_of(len(entries))
             if bucket not in self._graphs:
                 self._graphs[bucket] = DecodeGraph(self, bucket)
             logits = self._graphs[bucket].run(entries, marks[1] if marks else None)
         else:
+            if any(entry.source is not None for entry in entries):
+                raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
             ctx = self.build_context(entries)
             if marks:
                 marks[1].record()
@@ -216,7 +231,7 @@ class DecodeGraph:
         self.widths = [max(1, (longest + cache.page_size - 1) // cache.page_size) for _ in cache.groups]
         layout = [("tokens", (bucket,)), ("positions", (bucket,)), ("token_seq", (bucket,)), ("no_slots", (bucket,)),
                   ("seq_start", (bucket + 1,)), ("seq_first_pos", (bucket,)), ("seq_len", (bucket,)), ("seq_slot", (bucket,)),
-                  ("want_rows", (bucket,))]
+                  ("want_rows", (bucket,)), ("token_source", (bucket,))]
         for group, width in enumerate(self.widths):
             layout += [(f"block_table{group}", (bucket, width)), (f"slot_map{group}", (bucket,))]
         total = sum(int(np.prod(shape)) for _, shape in layout)
@@ -233,6 +248,10 @@ class DecodeGraph:
         self.host["seq_start"][:] = np.arange(bucket + 1)
         self.host["want_rows"][:] = np.arange(bucket)
         self.host["no_slots"][:] = -1
+        self.host["token_source"][:] = -1
+        self.token_source = views["token_source"]
+        self.copied = torch.cuda.Event()                    # the last transfer of the pinned buffer has been made
+        self.copy_pending = False
         groups = [GroupView(views[f"block_table{group}"], views[f"slot_map{group}"], width)
                   for group, width in enumerate(self.widths)]
         self.ctx = StepContext(
@@ -261,6 +280,8 @@ class DecodeGraph:
             host[name][count:stale] = 0
         host["seq_len"][count:stale] = 1
         host["tokens"][:count] = [int(entry.tokens[0]) for entry in entries]
+        host["token_source"][:count] = [-1 if entry.source is None else int(entry.source) for entry in entries]
+        host["token_source"][count:stale] = -1
         host["positions"][:count] = positions
         host["seq_first_pos"][:count] = positions
         host["seq_len"][:count] = [position + 1 for position in positions]
@@ -292,8 +313,16 @@ class DecodeGraph:
     def run(self, entries: Sequence[StepEntry], transferred=None) -> torch.Tensor:
         """`transferred`: an event to record once the step's arrays are on their way."""
         runner = self.runner
+        if self.copy_pending:
+            # the pinned buffer is written again only after its last transfer has read it (a caller
+            # may run steps without ever waiting for one)
+            self.copied.synchronize()
         self._fill(entries)
         self.device_flat.copy_(self.pinned, non_blocking=True)
+        self.copied.record()
+        self.copy_pending = True
+        if any(entry.source is not None for entry in entries):
+            ops_feed_tokens(self.ctx.tokens, self.token_source, runner.device_tokens)
         if transferred is not None:
             transferred.record()
         if self.graph is None:

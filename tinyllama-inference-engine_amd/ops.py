@@ -260,10 +260,12 @@ def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | Non
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
-           seed: torch.Tensor | None = None, counter: torch.Tensor | None = None) -> torch.Tensor:
+           seed: torch.Tensor | None = None, counter: torch.Tensor | None = None,
+           out: torch.Tensor | None = None) -> torch.Tensor:
     """One token per row of float32 logits: the first maximum when the row's temperature is not
     positive (or none is given), else a draw from the top-p part of softmax(logits / T) with the
-    uniform number of (seed, counter).  A row with a NaN or an infinity gives -1."""
+    uniform number of (seed, counter).  A row with a NaN or an infinity gives -1.  `out`: int32
+    [rows] to write into (else a new tensor)."""
     _device_tensor(logits, "logits", torch.float32)
     if logits.dim() != 2:
         raise invalid_shape("sample takes logits [rows, vocab]")
@@ -274,12 +276,29 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p:
             _device_tensor(tensor, name, dtype)
             if tensor.shape != (rows,):
                 raise invalid_shape(f"sample: {name} needs one entry per row")
-    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    else:
+        _device_tensor(out, "out", torch.int32)
+        if out.shape != (rows,):
+            raise invalid_shape("sample: out needs one entry per row")
     if rows == 0:
         return out
     _check(library().tlie_sample(_ptr(logits), rows, logits.shape[1], _ptr(temperature), _ptr(top_p), _ptr(seed),
                                  _ptr(counter), _ptr(out), _stream()), "sample")
     return out
+
+
+def feed_tokens(tokens: torch.Tensor, source: torch.Tensor, sampled: torch.Tensor) -> None:
+    """tokens[i] = sampled[source[i]] wherever source[i] >= 0, on the device.  The caller has
+    checked on the host that every such source is a row of `sampled`."""
+    for name, tensor in (("tokens", tokens), ("source", source), ("sampled", sampled)):
+        _device_tensor(tensor, name, torch.int32)
+    if tokens.dim() != 1 or source.shape != tokens.shape or sampled.dim() != 1 or sampled.shape[0] == 0:
+        raise invalid_shape("feed_tokens takes tokens [T], source [T] and sampled [rows]")
+    if tokens.shape[0] == 0:
+        return
+    _check(library().tlie_feed_tokens(_ptr(tokens), _ptr(source), _ptr(sampled), tokens.shape[0], _stream()), "feed_tokens")
 
 
 # ---- bfloat16 kernels on the matrix cores ---------------------------------------------------------
