@@ -350,7 +350,7 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
         assert torch.equal(decode, out)
         # several waves of a workgroup sharing the keys: the same result within rounding (the sums run in another order)
         waves = 2
-        while waves <= 16 and waves * d <= 1024:
+        while waves <= ops.attention_max_waves(d):
             shared = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
                                         1.0 / math.sqrt(d), nsplit, split_len, 1, waves)
             assert rel_err(shared, out.double()) < 1e-2, f"{waves} waves"
@@ -370,6 +370,7 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     dict(tokens=97, nq=7, nkv=7, d=112, page=16),
 ])
 def test_attention_mfma(case):
+    from tlie_amd import ops
     tokens, nq, nkv, d, page = case["tokens"], case["nq"], case["nkv"], case["d"], case["page"]
     window = case.get("window")
     torch.manual_seed(tokens)
@@ -384,7 +385,7 @@ def test_attention_mfma(case):
     # 2 and 4 waves of a workgroup share each tile's keys (whole and in 3 parts), the tiles longest first
     for waves, nsplit in ((2, 1), (4, 1), (4, 3)):
         col_tiles = 2 if d <= 128 else 1
-        if waves * col_tiles * d <= 1024:
+        if waves <= ops.attention_max_waves(d, col_tiles):
             shared = run_attention_mfma(q, k, v, page, window, nsplit, shuffle_seed=tokens, col_tiles=col_tiles, waves=waves)
             assert rel_err(shared, want) < TOL["bfloat16"], f"{waves} waves, {nsplit} parts"
     # the last token alone (a decode step), its key range cut in parts that are merged

@@ -72,10 +72,16 @@ __device__ __forceinline__ float groups_sum(float v) {
 // sequence * ceil(G / 16) + tile of the group.
 // DT = head_dim / 16.  CT = groups of 16 columns per wave: a tile has 16 * CT columns, and every
 // key and value the wave loads serves all of them (prompt portions take CT = 4, decode steps 1).
-// A workgroup has at most 1024 / (16 * CT * DT) waves (16 at most): their merge fits LDS, and the
-// compiler may give each wave the registers that leaves.
+// A workgroup has at most 8 waves, and at most 1024 / (16 * CT * DT): their merge fits LDS, and
+// every wave may use 256 registers;
+// head sizes above 128 need more registers still and get 4 waves at most.
+constexpr int attention_max_waves(int dt, int ct) {
+  const int fit = 1024 / (16 * ct * dt), cap = dt * ct > 8 ? 4 : 8;
+  return fit > cap ? cap : (fit < 1 ? 1 : fit);
+}
+
 template <int DT, int CT>
-__global__ void __launch_bounds__(64 * (1024 / (16 * CT * DT) > 16 ? 16 : (1024 / (16 * CT * DT) < 1 ? 1 : 1024 / (16 * CT * DT))))
+__global__ void __launch_bounds__(64 * attention_max_waves(DT, CT))
 attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache,
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
@@ -282,8 +288,14 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     }
   };
 
-  // Two blocks in turn: while one is worked on, the other is on its way.  Without a window the
-  // first block's place is known before the position is: split_lo & ~31.
+  // A ring of blocks: while one is worked on, the others are on their way: four with one column
+  // group a wave and a head size up to 64 (a decode step lives on the loads it has in flight:
+  // inside whole decode steps of the TinyLlama shape four measured 1.5% faster than two at batch
+  // 1, 8 and 64), two otherwise, the registers hold no more.  The ring's first loads are made
+  // before the sequence's length is known (without a window the first block's place is
+  // split_lo & ~31 whatever the position), so some may lie past the range: they are safe (see
+  // above) and unused.  Later ones are made only inside the range.
+  constexpr int NB = (CT == 1 && DT <= 4) ? 4 : 2;
   const int first_block = ((window > 0 ? range_lo : split_lo) & ~31) + 32 * wave;
   const int stride = 32 * waves;
   // a block that every column of the tile sees whole: inside the range, below the first column's
@@ -296,14 +308,17 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     else
       work_block(kb, block, std::true_type{});
   };
-  KeyBlock even, odd;
-  load_block(first_block, even);
-  for (int kb = first_block; kb < range_hi; kb += 2 * stride) {
-    load_block(kb + stride, odd);
-    work(kb, even);
-    if (kb + stride >= range_hi) break;
-    load_block(kb + 2 * stride, even);
-    work(kb + stride, odd);
+  KeyBlock ring[NB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) load_block(first_block + j * stride, ring[j]);
+  for (int kb = first_block; kb < range_hi; kb += NB * stride) {
+#pragma unroll
+    for (int j = 0; j < NB; ++j) {
+      const int mine = kb + j * stride;
+      if (mine >= range_hi) break;
+      work(mine, ring[j]);
+      if (mine + NB * stride < range_hi) load_block(mine + NB * stride, ring[j]);
+    }
   }
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) running_sum[ct] = groups_sum(running_sum[ct]);
@@ -454,7 +469,8 @@ using namespace tlie;
 // part_o: float [tokens * nq * nsplit * d], part_ml: float [tokens * nq * nsplit * 2] (both only when nsplit > 1);
 // split_len: positions per part, a multiple of 32, nsplit * split_len >= the longest sequence.
 // d % 16 == 0, d <= 256, page_size a power of two >= 16; col_tiles 1, or 4 for d <= 64, or 2 for d <= 128.
-// waves: 1, 2, 4, 8 or 16 waves of a workgroup share a tile's keys; waves * col_tiles * d <= 1024 (their merge's LDS).
+// waves: 1, 2, 4 or 8 waves of a workgroup share a tile's keys; waves * col_tiles * d <= 1024 (their merge's LDS), and
+// at most 4 when col_tiles * d > 128.
 extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
                                    const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                                    float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
@@ -464,7 +480,7 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
     return kBadArgument;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr || split_len <= 0 || split_len % 32 != 0)) return kBadArgument;
   if (col_tiles != 1 && !(col_tiles == 4 && d <= 64) && !(col_tiles == 2 && d <= 128)) return kBadArgument;
-  if (waves < 1 || waves > 16 || (waves & (waves - 1)) != 0 || (waves > 1 && waves * col_tiles * d > 1024)) return kBadArgument;
+  if (waves < 1 || (waves & (waves - 1)) != 0 || waves > attention_max_waves(d / 16, col_tiles)) return kBadArgument;
   if (tiles == nullptr && (col_tiles != 1 || num_tiles != tokens * ((nq / nkv + 15) / 16))) return kBadArgument;
   if (!(scale > 0.f)) return kBadArgument;     // the maximum is taken before the scores are scaled
   hipStream_t s = (hipStream_t)stream;

@@ -82,6 +82,7 @@ class StepContext:
         batch 64 and 2048 positions 4 parts reach 5 TB/s, 16 parts 4 TB/s, and merging more than 16
         costs more than it gains), each part a multiple of 32 positions and at least 64.
         Returns (tiles, col_tiles, nsplit, split_len, waves of a workgroup that share a tile's keys)."""
+        from ..ops import attention_max_waves
         decode = self.max_new == 1 and self.num_seqs == self.num_tokens
         col_tiles = 1
         if decode:
@@ -102,7 +103,7 @@ class StepContext:
             # the step waits for (a prompt of 2048 tokens: 70 us against 87 with one wave a tile)
             nsplit = max(1, min((512 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
             waves = 1
-            while (waves < 4 and waves * 2 * col_tiles * head_dim <= 1024
+            while (waves < 4 and waves * 2 <= attention_max_waves(head_dim, col_tiles)
                    and self.max_context >= nsplit * waves * 2 * 128):
                 waves *= 2
         else:
@@ -111,7 +112,7 @@ class StepContext:
             # launch, while a wave keeps 128 keys or more
             nsplit = max(1, min((256 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
             waves = 1
-            while (waves < 4 and waves * 2 * head_dim <= 1024 and tiles_all * nsplit * waves * 2 <= 1024
+            while (waves < 4 and waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 1024
                    and self.max_context >= nsplit * waves * 2 * 128):
                 waves *= 2
         if nsplit == 1:

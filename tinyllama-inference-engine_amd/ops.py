@@ -358,6 +358,12 @@ def attention_col_tiles(head_dim: int) -> int:
     return 2 if head_dim <= 128 else 1
 
 
+def attention_max_waves(head_dim: int, col_tiles: int = 1) -> int:
+    """How many waves of a workgroup of the tiled attention kernel may share a tile's keys."""
+    fit, cap = 1024 // (col_tiles * head_dim), 4 if col_tiles * head_dim > 128 else 8
+    return max(1, min(fit, cap))
+
+
 def attention_tiles(seq_start, groups_per_kv: int, col_tiles: int = 1, seq_len=None):
     """The work list of the tiled attention kernel for a step, on the host: for every sequence,
     tiles of 16 * col_tiles columns, a column being a (token, query head of one group) pair.
@@ -395,7 +401,7 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     a decode step, in which token i is the one token of sequence i.  nsplit > 1 cuts the keys into
     that many parts of split_len positions (a multiple of 32; nsplit * split_len must reach the
     longest sequence) that run side by side and are merged.  col_tiles: the value the tiles were
-    made with.  waves (a power of two up to 16, waves * col_tiles * d <= 1024): so many waves of a
+    made with.  waves (a power of two up to `attention_max_waves`): so many waves of a
     workgroup share each tile's (or part's) keys and merge their results before writing."""
     _device_tensor(q, "q", torch.bfloat16)
     _device_tensor(cache, "cache", torch.bfloat16)
@@ -425,8 +431,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
         num_tiles = tokens * ((num_heads // num_kv_heads + 15) // 16)
     if nsplit > 1 and (split_len <= 0 or split_len % 32 != 0):
         raise invalid_argument("attention: split_len must be a positive multiple of 32")
-    if waves not in (1, 2, 4, 8, 16) or (waves > 1 and waves * col_tiles * head_dim > 1024):
-        raise invalid_argument("attention: waves must be a power of two up to 16 with waves * col_tiles * d <= 1024")
+    if waves not in (1, 2, 4, 8) or waves > attention_max_waves(head_dim, col_tiles):
+        raise invalid_argument(f"attention: waves must be a power of two up to {attention_max_waves(head_dim, col_tiles)}")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
         raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a power of two of rows (at least 16)")
     out = torch.empty_like(q)
