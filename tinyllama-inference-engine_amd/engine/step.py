@@ -109,10 +109,12 @@ class StepContext:
         else:
             # workgroups share a tile's keys until there is one for every compute unit (their sums
             # meet in the merge kernel); then the waves of a workgroup share them, which costs no
-            # launch, while a wave keeps 128 keys or more
+            # launch, while a wave keeps 128 keys or more and the step has 2048 waves at most
+            # (measured inside whole steps at 2048 positions: batch 1 16 parts x 1 wave, batch 8
+            # 8 x 2, batch 64 1 x 8)
             nsplit = max(1, min((256 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
             waves = 1
-            while (waves < 4 and waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 1024
+            while (waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 2048
                    and self.max_context >= nsplit * waves * 2 * 128):
                 waves *= 2
         if nsplit == 1:
