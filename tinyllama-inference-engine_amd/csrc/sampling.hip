@@ -38,6 +38,22 @@ __device__ __forceinline__ float uniform01(uint64_t seed, uint64_t counter) {
 
 constexpr int kSampleThreads = 1024;
 
+// f(index, value) for every element of the row, spread over the block's threads; a thread meets its
+// indices in rising order.  Rows that start on a 16-byte boundary are read four elements at a time.
+template <typename F>
+__device__ __forceinline__ void scan_row(const float* __restrict__ row, int vocab, int tid, F f) {
+  int done = 0;
+  if ((reinterpret_cast<uintptr_t>(row) & 15) == 0) {
+    const int chunks = vocab >> 2;
+    for (int c = tid; c < chunks; c += kSampleThreads) {
+      const float4 v = reinterpret_cast<const float4*>(row)[c];
+      f(4 * c, v.x), f(4 * c + 1, v.y), f(4 * c + 2, v.z), f(4 * c + 3, v.w);
+    }
+    done = chunks << 2;
+  }
+  for (int i = done + tid; i < vocab; i += kSampleThreads) f(i, row[i]);
+}
+
 // out[r] = sampled token, or -1 when the row holds a NaN or an infinity.
 __global__ void __launch_bounds__(kSampleThreads)
 sample_kernel(const float* __restrict__ logits, int vocab, const float* __restrict__ temperature,
@@ -54,11 +70,10 @@ sample_kernel(const float* __restrict__ logits, int vocab, const float* __restri
   float best = -INFINITY;
   int best_index = 0x7fffffff;
   int bad = 0;
-  for (int i = tid; i < vocab; i += kSampleThreads) {
-    const float v = row[i];
+  scan_row(row, vocab, tid, [&](int i, float v) {
     if (!isfinite(v)) bad = 1;
-    if (v > best) { best = v; best_index = i; }     // strided scan: a thread meets its indices in rising order
-  }
+    if (v > best) { best = v; best_index = i; }     // a thread meets its indices in rising order
+  });
   const float row_max = block_max(best, scratch);
   const int any_bad = __syncthreads_or(bad);
   // first index among the threads that hold the maximum
@@ -81,7 +96,7 @@ sample_kernel(const float* __restrict__ logits, int vocab, const float* __restri
   const float p_keep = top_p ? top_p[r] : 1.f;
 
   float local = 0.f;
-  for (int i = tid; i < vocab; i += kSampleThreads) local += expf((row[i] - row_max) * inv_temp);
+  scan_row(row, vocab, tid, [&](int, float v) { local += expf((v - row_max) * inv_temp); });
   const float total = block_sum(local, scratch);
 
   uint32_t threshold = 0;        // keep every token whose key is >= threshold
@@ -90,10 +105,9 @@ sample_kernel(const float* __restrict__ logits, int vocab, const float* __restri
     for (int bit = 31; bit >= 0; --bit) {
       const uint32_t trial = threshold | (1u << bit);
       float mass = 0.f;
-      for (int i = tid; i < vocab; i += kSampleThreads) {
-        const float v = row[i];
+      scan_row(row, vocab, tid, [&](int, float v) {
         if (order_key(v) >= trial) mass += expf((v - row_max) * inv_temp);
-      }
+      });
       mass = block_sum(mass, scratch);
       if (mass >= target) threshold = trial;
     }
