@@ -286,6 +286,15 @@ def test_replay_program_and_command_line(setups, tmp_path):
     assert_close(step1, plain_logits(setup, other)[[20]], TOLERANCE["float32"], "step 1")
     assert_close(step2, want[[39]], TOLERANCE["float32"], "step 2")
 
+    # what is no step, or ends a request that is not live, is an error line and exit status 1; the steps before it stand
+    for bad_line, code in (('{"step": 7, "entries": [{"id": "a", "tokens": "x"}]}', "invalid_argument"), ("not json", "invalid_argument"),
+                           ('{"step": 7, "entries": [], "end": ["nobody"]}', "invalid_argument"),
+                           ('{"step": 7, "entries": [{"id": "a", "tokens": [999999], "want": [0]}]}', "out_of_bounds")):
+        run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", setup["folder"], "--dtype", "float32",
+                              "--out", str(tmp_path / "bad"), "--max-tokens", "128"], input=json.dumps(lines[0]) + "\n" + bad_line + "\n",
+                             capture_output=True, text=True, timeout=300)
+        assert run.returncode == 1 and run.stdout.split() == ["done", "0"] and error_code(run.stderr) == code, (bad_line, run.stderr)
+
     prompt = "ids:" + ",".join(str(token) for token in tokens[:9])
     cli = [sys.executable, os.path.join(ROOT, "bin", "tinyllama_amd")]
     run = subprocess.run(cli + ["generate", setup["folder"], prompt, "6", "--dtype", "float32"], capture_output=True, text=True, timeout=300)
