@@ -59,27 +59,42 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[r][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  for (int c0 = k_begin; c0 < k_end; c0 += CHUNK) {
+  // Two sets of operand registers in turn: the next chunk's part of W, and its part of x, are asked
+  // for before the current chunk is multiplied, so that memory and the matrix cores work at once.
+  constexpr int kVectors = CHUNK / 8;                                  // 16-byte pieces of a staged row of x
+  constexpr int kStage = (NT * 16 * kVectors + kSkinnyThreads - 1) / kSkinnyThreads;   // pieces a thread stages
+  Pack16 a[2][RS][kSteps][2];
+  uint4 staged[kStage];
+  auto load_w = [&](int c0, Pack16 (&buf)[RS][kSteps][2]) {
     const int c1 = min(k_end, c0 + CHUNK);
-    // this wave's part of W for the chunk: issued first, in flight while x is staged
-    Pack16 a[RS][kSteps][2];
 #pragma unroll
     for (int r = 0; r < RS; ++r)
 #pragma unroll
       for (int s = 0; s < kSteps; ++s) {
         const int k = c0 + s * 64 + group * 16;
-        a[r][s][0].u = (active[r] && k < c1) ? *reinterpret_cast<const uint4*>(w_row[r] + k) : make_uint4(0, 0, 0, 0);
-        a[r][s][1].u = (active[r] && k + 8 < c1) ? *reinterpret_cast<const uint4*>(w_row[r] + k + 8) : make_uint4(0, 0, 0, 0);
+        buf[r][s][0].u = (active[r] && k < c1) ? *reinterpret_cast<const uint4*>(w_row[r] + k) : make_uint4(0, 0, 0, 0);
+        buf[r][s][1].u = (active[r] && k + 8 < c1) ? *reinterpret_cast<const uint4*>(w_row[r] + k + 8) : make_uint4(0, 0, 0, 0);
       }
-    __syncthreads();                         // the previous chunk's reads of xs are done
-    constexpr int kVectors = CHUNK / 8;
-    for (int i = threadIdx.x; i < NT * 16 * kVectors; i += kSkinnyThreads) {
+  };
+  auto load_x = [&](int c0) {
+    const int c1 = min(k_end, c0 + CHUNK);
+#pragma unroll
+    for (int j = 0; j < kStage; ++j) {
+      const int i = threadIdx.x + j * kSkinnyThreads;
       const int token = i / kVectors, k = c0 + (i % kVectors) * 8;
-      uint4 value = make_uint4(0, 0, 0, 0);
-      if (token < M && k < c1) value = *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * K + k);
-      *reinterpret_cast<uint4*>(xs + token * kStride + (k - c0)) = value;
+      staged[j] = (token < M && k < c1) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * K + k)
+                                        : make_uint4(0, 0, 0, 0);
     }
-    __syncthreads();
+  };
+  auto store_x = [&]() {
+#pragma unroll
+    for (int j = 0; j < kStage; ++j) {
+      const int i = threadIdx.x + j * kSkinnyThreads;
+      if (i < NT * 16 * kVectors) *reinterpret_cast<uint4*>(xs + (i / kVectors) * kStride + (i % kVectors) * 8) = staged[j];
+    }
+  };
+  auto multiply = [&](int c0, Pack16 (&buf)[RS][kSteps][2]) {
+    const int c1 = min(k_end, c0 + CHUNK);
 #pragma unroll
     for (int s = 0; s < kSteps; ++s) {
       if (c0 + s * 64 >= c1) break;          // the same for every lane
@@ -92,10 +107,27 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
         b1.u = *reinterpret_cast<const uint4*>(x_row + 8);
 #pragma unroll
         for (int r = 0; r < RS; ++r) {
-          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[r][s][0].v, b0.v, acc[r][t], 0, 0, 0);
-          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[r][s][1].v, b1.v, acc[r][t], 0, 0, 0);
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[r][s][0].v, b0.v, acc[r][t], 0, 0, 0);
+          acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(buf[r][s][1].v, b1.v, acc[r][t], 0, 0, 0);
         }
       }
+    }
+  };
+  load_w(k_begin, a[0]);
+  load_x(k_begin);
+  for (int c0 = k_begin; c0 < k_end; c0 += 2 * CHUNK) {
+#pragma unroll
+    for (int turn = 0; turn < 2; ++turn) {
+      const int mine = c0 + turn * CHUNK;
+      if (mine >= k_end) break;
+      __syncthreads();                       // the previous chunk's reads of xs are done
+      store_x();
+      __syncthreads();
+      if (mine + CHUNK < k_end) {
+        load_w(mine + CHUNK, a[turn ^ 1]);
+        load_x(mine + CHUNK);
+      }
+      multiply(mine, a[turn]);
     }
   }
   // acc[r][t][j] = y[token t*16 + (lane & 15)][wave_row + r*16 + group*4 + j]
