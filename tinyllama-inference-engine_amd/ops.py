@@ -304,21 +304,19 @@ def feed_tokens(tokens: torch.Tensor, source: torch.Tensor, sampled: torch.Tenso
 # ---- bfloat16 kernels on the matrix cores ---------------------------------------------------------
 SKINNY_MAX_ROWS = 64
 def skinny_split_len(rows: int, out_features: int, in_features: int) -> int:
-    """How many k values one split takes.  Measured on the MI355X over the TinyLlama shapes: a
-    workgroup that streams 256 to 512 k values of its 64 rows is fastest at every batch size;
-    longer splits leave the 256 CUs with too few workgroups to hide the first load's latency,
-    shorter ones pay more in partial sums than they gain.  Matrices with many rows (the gated
-    feed-forward's first product, the output head) take the longer splits, and more rows of x
-    take longer ones still, because each partial sum is a write and a read of rows x outputs."""
+    """How many k values one split takes.  Measured on the MI355X inside whole decode steps of the
+    TinyLlama shapes: matrices of few rows (2048, 2560) are fastest with 256 k values a workgroup
+    (longer splits leave the 256 CUs too few workgroups); the gated feed-forward's first product
+    (11264 rows) with 512, and 1024 once the step has more than 32 rows of x, because each partial
+    sum is a write and a read of rows x outputs; a long inner size (5632) with 1024 up to 32 rows
+    and 512 beyond."""
     strips = (out_features + 15) // 16
-    if rows > 16 and strips >= 1024:
-        length = 1024
-    elif strips >= 512:
-        length = 512
+    if strips >= 512:
+        length = 1024 if rows > 32 else 512
     else:
         length = 256
     if in_features >= 4096:
-        length = max(length, 512)            # a long inner size would leave its consumer too many partial sums
+        length = max(length, 1024 if rows <= 32 else 512)
     return min(length, (in_features + 63) // 64 * 64)
 
 
