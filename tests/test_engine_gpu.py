@@ -476,3 +476,38 @@ def test_a_request_that_stops_at_a_token_beside_one_that_does_not(setups):
     assert other.generated == free[1] and other.finish_reason == "length"
     assert 0 < engine.stats["steps_ahead"] <= engine.stats["steps"] - len(want)
     assert engine.cache.free_pages() == [engine.cache.num_pages]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype):
+    """The same check for steps of 17 to 24 requests, which take other kernels than small steps do
+    (products that leave partial sums to their consumers): every replay of the recording against
+    the same step launched kernel by kernel, requests ending mid-way."""
+    setup = setups("B", dtype)
+    recorded, eager = new_engine(setup, dtype, max_tokens=2048, max_requests=24), \
+        new_engine(setup, dtype, max_tokens=2048, max_requests=24, use_graphs=False)
+    prompts = {f"m{i}": request_tokens("B", 300 + i, 3 + (7 * i) % 23) for i in range(24)}
+    follow = {request: request_tokens("B", 400 + i, 12) for i, request in enumerate(prompts)}
+    a, b = Replayer(recorded), Replayer(eager)
+    for replay in (a, b):
+        replay.step([(request, tokens, [len(tokens) - 1]) for request, tokens in prompts.items()])
+    live = list(prompts)
+    for turn in range(12):
+        if turn in (4, 8):
+            for request in live[5:8]:
+                for replay in (a, b):
+                    replay.engine.finish(request)
+            del live[5:8]
+        items = [(request, [follow[request][turn]], [0]) for request in live]
+        a.step(items)
+        b.step(items)
+        torch.cuda.synchronize()
+    assert 32 in recorded.runner._graphs and recorded.runner._graphs[32].graph is not None
+    keys = sorted(a.rows, key=str)
+    assert keys == sorted(b.rows, key=str)
+    got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
+    bad = first_bad_row(got, want, CUT_TOLERANCE[dtype])
+    assert bad is None, f"replayed step differs from the eager one at {keys[bad]}"
+    plain = plain_logits(setup, prompts["m3"] + follow["m3"])
+    mine = torch.stack([a.rows[("m3", position)] for position in range(len(prompts["m3"]) - 1, len(prompts["m3"]) + 12)])
+    assert first_bad_row(mine, plain[len(prompts["m3"]) - 1:], TOLERANCE[dtype]) is None

@@ -77,7 +77,10 @@ class Product:
 
     def dense(self, dtype: torch.dtype | None = None) -> torch.Tensor:
         """The summed result as one tensor (for parts that do not fuse the sum)."""
-        out = self.data if self.nsplit == 1 and self.data.dim() == 2 else self.data.view(self.nsplit, self.rows, self.cols).sum(0)
+        if self.nsplit == 1:
+            out = self.data.view(self.rows, self.cols)        # nothing to add up: no kernel runs
+        else:
+            out = self.data.view(self.nsplit, self.rows, self.cols).sum(0)
         return out if dtype is None or out.dtype == dtype else out.to(dtype)
 
 
