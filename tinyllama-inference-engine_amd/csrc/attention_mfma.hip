@@ -294,7 +294,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   // 1, 8 and 64), two otherwise, the registers hold no more.  The ring's first loads are made
   // before the sequence's length is known (without a window the first block's place is
   // split_lo & ~31 whatever the position), so some may lie past the range: they are safe (see
-  // above) and unused.  Later ones are made only inside the range.
+  // above) and unused.
   constexpr int NB = (CT == 1 && DT <= 4) ? 4 : 2;
   const int first_block = ((window > 0 ? range_lo : split_lo) & ~31) + 32 * wave;
   const int stride = 32 * waves;
@@ -317,7 +317,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
       const int mine = kb + j * stride;
       if (mine >= range_hi) break;
       work(mine, ring[j]);
-      if (mine + NB * stride < range_hi) load_block(mine + NB * stride, ring[j]);
+      // (a ring of two keeps asking past the range: the unconditional load measured 1.5% faster in
+      // prompt steps; a ring of four asks only inside the range, which measured 2% faster in decode steps)
+      if (NB == 2 || mine + NB * stride < range_hi) load_block(mine + NB * stride, ring[j]);
     }
   }
 #pragma unroll
