@@ -511,3 +511,29 @@ def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype):
     plain = plain_logits(setup, prompts["m3"] + follow["m3"])
     mine = torch.stack([a.rows[("m3", position)] for position in range(len(prompts["m3"]) - 1, len(prompts["m3"]) + 12)])
     assert first_bad_row(mine, plain[len(prompts["m3"]) - 1:], TOLERANCE[dtype]) is None
+
+
+def test_a_dropped_engine_frees_its_recordings_at_once(setups):
+    """An engine and its recorded steps must not be cyclic garbage: the cycle collector would free
+    them at a moment of its choosing, and inside another recording's capture the graph's destructor
+    ends the process.  Dropping the last reference frees them, with the collector switched off."""
+    import gc
+    import weakref
+    from tlie_amd import StepEntry
+    setup = setups("A", "bfloat16")
+    gc.collect()
+    gc.disable()
+    try:
+        engine = new_engine(setup, "bfloat16")
+        engine.admit("r")
+        engine.step([StepEntry("r", [1, 2, 3], [])])
+        for token in (4, 5, 6):
+            engine.step([StepEntry("r", [token], [0])])
+        recording = engine.runner._graphs[1]
+        assert recording.graph is not None
+        watched = [weakref.ref(engine), weakref.ref(engine.runner), weakref.ref(recording), weakref.ref(recording.graph)]
+        del recording
+        del engine
+        assert [watch() for watch in watched] == [None, None, None, None]
+    finally:
+        gc.enable()

@@ -10,6 +10,8 @@ after the step is enqueued.
 """
 from __future__ import annotations
 
+import gc
+import weakref
 from dataclasses import dataclass, field
 from typing import Hashable, Sequence
 
@@ -228,7 +230,12 @@ class DecodeGraph:
         return bucket
 
     def __init__(self, runner: "ModelRunner", bucket: int):
-        self.runner, self.bucket = runner, bucket
+        # The runner owns its recordings; a recording that owned its runner in turn would make the
+        # pair garbage that only the cycle collector frees, at a moment of its choosing: if that
+        # moment falls inside another recording's capture, the graph's destructor (which waits for
+        # the device) is an operation the capture forbids, and the process ends.
+        self._runner = weakref.ref(runner)
+        self.bucket = bucket
         cache = runner.cache
         longest = cache.max_positions or cache.num_pages * cache.page_size
         self.widths = [max(1, (longest + cache.page_size - 1) // cache.page_size) for _ in cache.groups]
@@ -267,6 +274,13 @@ class DecodeGraph:
         self.logits = None
         self._rows_filled = bucket                           # rows that may hold a step's values
         self._known = [[(0, 0)] * bucket for _ in cache.groups]   # per group and row: (admission, blocks written)
+
+    @property
+    def runner(self) -> "ModelRunner":
+        runner = self._runner()
+        if runner is None:
+            raise invalid_argument("the recording has outlived its runner")
+        return runner
 
     def _fill(self, entries: Sequence[StepEntry]) -> None:
         """The step's arrays in the pinned buffer.  A row's part of a block table is kept from
@@ -334,8 +348,18 @@ class DecodeGraph:
             logits = runner.model.forward(self.ctx, runner.cache.bindings)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self.logits = runner.model.forward(self.ctx, runner.cache.bindings)
+            # no garbage collection while the capture is open: collecting some dead object that
+            # holds device resources (another engine's recording, say) would call into the device
+            # in ways a capture forbids
+            gc.collect()
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self.logits = runner.model.forward(self.ctx, runner.cache.bindings)
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
             return logits[:len(entries)]
         self.graph.replay()
