@@ -590,3 +590,47 @@ def test_rotation_in_paired_order_and_inside_the_product(case):
         assert rel_err(fused_cache, plain_cache.double()) < 1e-2
         untouched = plain_cache == -3.0
         assert torch.equal(fused_cache[untouched], plain_cache[untouched])
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_attention_and_products_at_random_sizes(seed):
+    """Sizes drawn at random (head sizes in steps of 16, any number of heads and groups, pages of
+    16 to 64 rows, windows, key parts, waves; product sizes that are no multiples of the tiles):
+    a portion of a sequence and its last token through the tiled attention kernel, and the same
+    random product through both kernels for few rows."""
+    from tlie_amd import ops
+    rng = random.Random(seed)
+    torch.manual_seed(seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 256])
+    nkv, group = rng.randint(1, 4), rng.choice([1, 2, 3, 4, 5, 8, 17])
+    nq, tokens, page = nkv * group, rng.randint(1, 420), rng.choice([16, 32, 64])
+    window = rng.choice([None, None, rng.randint(1, 200)])
+    q, k, v = torch.randn(tokens, nq, d), torch.randn(tokens, nkv, d), torch.randn(tokens, nkv, d)
+    want = plain_attention(rounded(q, torch.bfloat16), rounded(k, torch.bfloat16), rounded(v, torch.bfloat16), window=window)
+    col_tiles = rng.choice([c for c in (1, 2, 4) if c * d <= 256])
+    waves = rng.choice([w for w in (1, 2, 4, 8) if w <= ops.attention_max_waves(d, col_tiles)])
+    nsplit = rng.choice([1, 1, 2, 3, 7])
+    first = rng.randint(0, tokens - 1)
+    count = rng.randint(1, tokens - first)
+    what = f"d={d} nq={nq} nkv={nkv} tokens={tokens} page={page} window={window} col_tiles={col_tiles} waves={waves} nsplit={nsplit}"
+    got = run_attention_mfma(q, k, v, page, window, nsplit, token_list=list(range(first, first + count)), shuffle_seed=seed,
+                             col_tiles=col_tiles, waves=waves)
+    assert rel_err(got, want[first:first + count]) < TOL["bfloat16"], what
+    last = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=seed)
+    assert rel_err(last[0], want[-1]) < TOL["bfloat16"], what
+
+    m, n, inner = rng.randint(1, 64), rng.choice([rng.randint(1, 300), 2 * rng.randint(1, 2000)]), 8 * rng.randint(1, 700)
+    x, w, b = torch.randn(m, inner).bfloat16(), (torch.randn(n, inner) / math.sqrt(inner)).bfloat16(), torch.randn(n).bfloat16()
+    want = plain_linear(x.double(), w.double(), b.double())
+    what = f"m={m} n={n} k={inner}"
+    got = ops.gemm_skinny(x.to(DEV), w.to(DEV), b.to(DEV), split_len=rng.choice([None, 64, 128, 512])).dense()
+    assert rel_err(got, want) < 1e-5, what
+    if m <= 16:
+        waves = rng.choice([2, 4, 8, 16])
+        rows_per_block = rng.choice([8, 16, 32] if waves <= 8 else [8, 16])
+        got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), waves=waves, rows_per_block=rows_per_block).dense()
+        assert rel_err(got, want) < 1e-5, (what, waves, rows_per_block)
+        if n % 2 == 0:
+            full = plain_linear(x.double(), w.double())
+            act = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "silu", waves=waves, rows_per_block=rows_per_block)
+            assert rel_err(act, plain_silu_mul(full[:, 0::2], full[:, 1::2])) < TOL["bfloat16"], (what, waves, rows_per_block)
