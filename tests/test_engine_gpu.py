@@ -537,3 +537,33 @@ def test_a_dropped_engine_frees_its_recordings_at_once(setups):
         assert [watch() for watch in watched] == [None, None, None, None]
     finally:
         gc.enable()
+
+
+def test_long_prompts_take_the_walk_through_lds(tmp_path):
+    """A sequence long enough (1536 positions and more) that prompt portions are attended with
+    the keys brought through LDS once for four waves: the whole prompt, and the same in two
+    portions beside another request, against the plain implementation."""
+    raw = dict(CONFIGS["A"], max_position_embeddings=2048, num_hidden_layers=1)
+    folder = make_model(tmp_path / "model", raw, seed=21, dtype_name="bfloat16")
+    stored, weights = load_plain(folder)
+    length = 1800
+    tokens = random_tokens(5, length, raw["vocab_size"])
+    want = plain_forward(stored, weights, tokens)
+    from tlie_amd import Engine, StepEntry
+    engine = Engine(folder, dtype="bfloat16", max_tokens=4096, page_size=16, max_requests=4)
+    replay = Replayer(engine)
+    replay.step([("w", tokens, list(range(0, length, 7)) + [length - 1])], end=["w"])
+    places = list(range(0, length, 7)) + [length - 1]
+    bad = first_bad_row(replay.logits_of("w", places), want[places], TOLERANCE["bfloat16"])
+    assert bad is None, f"whole: first wrong position {places[bad]}"
+    other = random_tokens(6, 40, raw["vocab_size"])
+    replay.step([("p", tokens[:1000], []), ("o", other, [39])])
+    replay.step([("o", [3], [0]), ("p", tokens[1000:], list(range(800)))], end=["o", "p"])
+    bad = first_bad_row(replay.logits_of("p", range(1000, length)), want[1000:], TOLERANCE["bfloat16"])
+    assert bad is None, f"second portion: first wrong position {1000 + bad}"
+    # the step's policy did choose that walk
+    engine.admit("check")
+    engine.cache.reserve("check", 1700)
+    policy = engine.runner.build_context([StepEntry("check", tokens[:1700], [])]).attention_tiles(2, 2, 16)
+    assert policy[5] is True and policy[4] == 4
+    engine.finish("check")

@@ -320,9 +320,10 @@ def test_gemm_skinny_refuses():
     assert not ops.gemm_skinny_takes(torch.randn(2, 12, device=DEV).bfloat16(), torch.randn(8, 12, device=DEV).bfloat16())
 
 
-def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0, col_tiles=None, waves=1):
+def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_seed=0, col_tiles=None, waves=1, shared=False):
     """One sequence through the tiled kernel: q rows for the positions in token_list (default all).
-    waves > 1: so many waves share each tile's keys, and the tiles come longest first."""
+    waves > 1: so many waves share each tile's keys, and the tiles come longest first.  shared: the
+    waves take columns of their own instead, and the keys reach them through LDS."""
     from tlie_amd import ops
     import numpy as np
     tokens, nq, d = q.shape
@@ -333,7 +334,7 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     assert token_list == list(range(token_list[0], token_list[0] + len(token_list)))
     table = torch.tensor([[0] * len(pages), pages], dtype=torch.int32, device=DEV)
     col_tiles = col_tiles or ops.attention_col_tiles(d)
-    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv, col_tiles,
+    tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv, col_tiles * (waves if shared else 1),
                                 np.asarray([token_list[-1] + 1]) if waves > 1 else None)
     if waves > 1 and tiles.shape[0] > 1:
         assert tiles[0, 3] > tiles[-1, 3]                                      # the tile of the last tokens first
@@ -342,7 +343,7 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     rows = q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV)
     positions = torch.tensor(token_list, dtype=torch.int32, device=DEV)
     out = ops.attention_mfma(rows, cache.to(DEV), table, torch.from_numpy(tiles).to(DEV), positions, nq, nkv, d, window,
-                             1.0 / math.sqrt(d), nsplit, split_len, col_tiles, waves)
+                             1.0 / math.sqrt(d), nsplit, split_len, col_tiles, waves, shared)
     if len(token_list) == 1 and waves == 1:
         # the same step as a decode step: no work list, the kernel derives the tiles; the sequence must be row 0
         decode = ops.attention_mfma(rows, cache.to(DEV), table[1:].contiguous(), None, positions, nq, nkv, d, window,
@@ -388,6 +389,11 @@ def test_attention_mfma(case):
         if waves <= ops.attention_max_waves(d, col_tiles):
             shared = run_attention_mfma(q, k, v, page, window, nsplit, shuffle_seed=tokens, col_tiles=col_tiles, waves=waves)
             assert rel_err(shared, want) < TOL["bfloat16"], f"{waves} waves, {nsplit} parts"
+    # the waves of a workgroup take columns of their own, keys and values reach them through LDS
+    if d <= 128:
+        for waves, nsplit in ((4, 1), (8, 1), (4, 3)):
+            through_lds = run_attention_mfma(q, k, v, page, window, nsplit, shuffle_seed=tokens, col_tiles=2, waves=waves, shared=True)
+            assert rel_err(through_lds, want) < TOL["bfloat16"], f"through LDS, {waves} waves, {nsplit} parts"
     # the last token alone (a decode step), its key range cut in parts that are merged
     for nsplit in (1, 2, 5):
         last = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=tokens)
@@ -396,6 +402,10 @@ def test_attention_mfma(case):
     first, count = max(0, tokens // 2 - 9), min(21, tokens - max(0, tokens // 2 - 9))
     portion = run_attention_mfma(q, k, v, page, window, 1, token_list=list(range(first, first + count)), shuffle_seed=tokens)
     assert rel_err(portion, want[first:first + count]) < TOL["bfloat16"]
+    if d <= 128:
+        portion = run_attention_mfma(q, k, v, page, window, 1, token_list=list(range(first, first + count)), shuffle_seed=tokens,
+                                     col_tiles=2, waves=4, shared=True)
+        assert rel_err(portion, want[first:first + count]) < TOL["bfloat16"], "a portion through LDS"
     split_portion = run_attention_mfma(q, k, v, page, window, 3, token_list=list(range(first, first + count)), shuffle_seed=tokens)
     assert rel_err(split_portion, want[first:first + count]) < TOL["bfloat16"]
 

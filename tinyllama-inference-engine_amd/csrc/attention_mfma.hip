@@ -80,8 +80,12 @@ constexpr int attention_max_waves(int dt, int ct) {
   return fit > cap ? cap : (fit < 1 ? 1 : fit);
 }
 
-template <int DT, int CT>
-__global__ void __launch_bounds__(64 * attention_max_waves(DT, CT))
+// SHARED: the waves of a workgroup do not share a tile's keys but take 16 * CT columns each of a
+// tile of 16 * CT * waves columns, and every block of keys and values is brought once, through LDS,
+// for all of them (prompt portions: the tiles of neighbouring tokens read the same keys, and read
+// each on its own they are bound by the L2's bandwidth, not by their arithmetic).
+template <int DT, int CT, bool SHARED>
+__global__ void __launch_bounds__(SHARED ? 512 : 64 * attention_max_waves(DT, CT))
 attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache,
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
@@ -109,6 +113,9 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   ntok = __builtin_amdgcn_readfirstlane(ntok), col0 = __builtin_amdgcn_readfirstlane(col0);
   const int pos0 = __builtin_amdgcn_readfirstlane(positions[tok0]);
   const int ncols = ntok * G;
+  const int group_col0 = col0;                                   // the workgroup's first column
+  if (SHARED) col0 += __builtin_amdgcn_readfirstlane(wave) * 16 * CT;
+  const bool wave_active = col0 < ncols;                         // (a shared tile's last waves may have no column)
   bool valid_col[CT];
   int tok[CT], head[CT], pos_col[CT], lo_col[CT];
 #pragma unroll
@@ -126,14 +133,31 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   const int tile_hi = pos0 + last_col / G + 1;
   const int tile_lo = window > 0 ? max(0, pos0 + col0 / G - window + 1) : 0;
   const int split_lo = nsplit > 1 ? split * split_len : 0;
-  const int range_lo = max(tile_lo, split_lo);
-  const int range_hi = nsplit > 1 ? min(tile_hi, split_lo + split_len) : tile_hi;
+  const int range_lo = wave_active ? max(tile_lo, split_lo) : 0;
+  const int range_hi = wave_active ? (nsplit > 1 ? min(tile_hi, split_lo + split_len) : tile_hi) : 0;
 
   // Pages hold a power of two of rows, at least 16, and blocks of 32 keys start at multiples of 32:
   // each half of a block (16 keys) lies on one page, the same for every lane.  So the page numbers
   // are scalars, and a lane's addresses are a scalar base plus an offset that never changes.
   const int page_shift = 31 - __clz(page_size), page_mask = page_size - 1;
   const int* pages = block_table + static_cast<size_t>(seq) * max_blocks;
+  // For the walk that brings blocks through LDS: the wave keeps 128 consecutive entries of the
+  // sequence's block table in two registers, one entry a lane each, loaded before it walks the
+  // blocks they cover, and reads page numbers from there, so that a block asked for ahead of its
+  // turn does not wait for a page number to come back from memory first.
+  int table_first = 0, table_low = 0, table_high = 0;
+  auto load_table = [&](int first_index) {
+    table_first = first_index;
+    table_low = pages[min(first_index + lane, max_blocks - 1)];
+    table_high = pages[min(first_index + 64 + lane, max_blocks - 1)];
+  };
+  auto page_of = [&](int index) -> int {                   // index: the same for every lane, within the window
+    const int place = index - table_first;
+    const int low = __builtin_amdgcn_readlane(table_low, place & 63);
+    const int high = __builtin_amdgcn_readlane(table_high, place & 63);
+    return place < 64 ? low : high;
+  };
+  const int table_span = 128 << page_shift;                // keys that one window covers
   const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * D;
   const uint16_t* k_base = cache + static_cast<size_t>(kvh) * page_size * D;
   const uint16_t* v_base = k_base + static_cast<size_t>(nkv) * page_size * D;
@@ -308,6 +332,105 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     else
       work_block(kb, block, std::true_type{});
   };
+  if constexpr (SHARED) {
+    // ---- every block once for the whole workgroup, through LDS ------------------------------------
+    // keys as [key][D + 8] (the padding spreads a strip's 16 rows over the banks), values as
+    // [dim][32 + 4]; two buffers in turn, so that one barrier a block is enough: a wave writes
+    // buffer b of block i + 1 only after the barrier of block i, which every wave reaches only
+    // after it has read buffer b for block i - 1.
+    constexpr int kKeyStride = D + 8, kValueStride = 36;
+    __shared__ __attribute__((aligned(16))) uint16_t lds_k[2][32 * kKeyStride];
+    __shared__ __attribute__((aligned(16))) uint16_t lds_v[2][D * kValueStride];
+    constexpr int kPieces = 32 * D / 8;                  // 16-byte pieces of a block of keys; of its values as well
+    constexpr int kStage = (kPieces + 255) / 256;        // pieces a thread brings (a workgroup has 256 or 512 threads)
+    const int group_last = min(group_col0 + 16 * CT * waves - 1, ncols - 1);
+    const int group_hi = pos0 + group_last / G + 1;
+    const int group_lo = window > 0 ? max(0, pos0 + group_col0 / G - window + 1) : 0;
+    const int all_lo = max(group_lo, split_lo);
+    const int all_hi = nsplit > 1 ? min(group_hi, split_lo + split_len) : group_hi;
+    // Blocks are asked for kAhead blocks before their turn and wait in registers: a workgroup walks
+    // its blocks one after the other, and the longest tile's walk is what a prompt step waits for.
+    constexpr int kAhead = DT <= 4 ? 4 : 2;                // (larger heads: the registers hold no more)
+    typedef uint32_t Piece __attribute__((ext_vector_type(4)));     // a native vector: it stays in registers
+    Piece staged_k[kAhead][kStage], staged_v[kAhead][kStage];
+    auto bring = [&](int kb, Piece (&keys)[kStage], Piece (&values)[kStage]) {
+      const int page_a = page_of(kb >> page_shift);
+      const int page_b = page_of((kb + 16) >> page_shift);
+#pragma unroll
+      for (int j = 0; j < kStage; ++j) {
+        // (threads beyond the block's pieces load the last piece again and do not store it: a load
+        // under a condition would hide from the compiler how many loads are on their way)
+        const int piece = min(static_cast<int>(threadIdx.x + j * blockDim.x), kPieces - 1);
+        const int key = piece / (D / 8), chunk = piece % (D / 8);
+        const size_t page = key < 16 ? page_a : page_b;
+        keys[j] = *reinterpret_cast<const Piece*>(k_base + page * page_stride + ((kb + key) & page_mask) * D + chunk * 8);
+        const int half = piece / (2 * D), rest = piece % (2 * D), dim = rest >> 1, part = rest & 1;
+        const size_t value_page = half == 0 ? page_a : page_b;
+        values[j] = *reinterpret_cast<const Piece*>(v_base + value_page * page_stride + (static_cast<size_t>(dim) << page_shift) +
+                                                    ((kb + half * 16) & page_mask) + part * 8);
+      }
+    };
+    auto put = [&](int buffer, const Piece (&keys)[kStage], const Piece (&values)[kStage]) {
+#pragma unroll
+      for (int j = 0; j < kStage; ++j) {
+        const int piece = threadIdx.x + j * blockDim.x;
+        if (piece < kPieces) {
+          const int key = piece / (D / 8), chunk = piece % (D / 8);
+          *reinterpret_cast<Piece*>(lds_k[buffer] + key * kKeyStride + chunk * 8) = keys[j];
+          const int half = piece / (2 * D), rest = piece % (2 * D), dim = rest >> 1, part = rest & 1;
+          uint2* place = reinterpret_cast<uint2*>(lds_v[buffer] + dim * kValueStride + half * 16 + part * 8);
+          place[0] = make_uint2(values[j].x, values[j].y);
+          place[1] = make_uint2(values[j].z, values[j].w);
+        }
+      }
+    };
+    auto take = [&](int buffer, KeyBlock& block) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          block.k[t][ks].u = has_dims(ks) ? *reinterpret_cast<const uint4*>(lds_k[buffer] + (t * 16 + col) * kKeyStride + ks * 32 + grp * 8)
+                                          : make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+          block.v[dt][t] = *reinterpret_cast<const uint2*>(lds_v[buffer] + (dt * 16 + col) * kValueStride + t * 16 + grp * 4);
+      }
+    };
+    // One turn of the ring, for a place in it that is known when the code is compiled (so that the
+    // waiting blocks stay in registers).  Every turn asks for a block and stores one, whether or
+    // not a block is left (past the last one it asks for the last one again): the number of loads
+    // on their way is then the same on every path, and a turn waits for its own block only.
+    auto turn = [&](auto place, int mine, int last) {
+      constexpr int j = decltype(place)::value;
+      put(j & 1, staged_k[j], staged_v[j]);
+      __syncthreads();
+      bring(min(mine + 32 * kAhead, last), staged_k[j], staged_v[j]);
+      if (mine <= last && mine + 32 > range_lo && mine < range_hi) {
+        KeyBlock block;
+        take(j & 1, block);
+        work(mine, block);
+      }
+    };
+    for (int begin = all_lo & ~31; begin < all_hi; begin += table_span) {
+      load_table(begin >> page_shift);
+      const int last = (min(all_hi, begin + table_span) - 1) & ~31;      // the window's last block of the range
+      bring(begin, staged_k[0], staged_v[0]);
+      bring(min(begin + 32, last), staged_k[1], staged_v[1]);
+      if constexpr (kAhead == 4) {
+        bring(min(begin + 64, last), staged_k[2], staged_v[2]);
+        bring(min(begin + 96, last), staged_k[3], staged_v[3]);
+      }
+      for (int kb = begin; kb <= last; kb += 32 * kAhead) {
+        turn(std::integral_constant<int, 0>{}, kb, last);
+        turn(std::integral_constant<int, 1>{}, kb + 32, last);
+        if constexpr (kAhead == 4) {
+          turn(std::integral_constant<int, 2>{}, kb + 64, last);
+          turn(std::integral_constant<int, 3>{}, kb + 96, last);
+        }
+      }
+      __syncthreads();                                       // (the next window's first block reuses buffer 0)
+    }
+  } else {
   KeyBlock ring[NB];
 #pragma unroll
   for (int j = 0; j < NB; ++j) load_block(first_block + j * stride, ring[j]);
@@ -322,10 +445,11 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
       if (NB == 2 || mine + NB * stride < range_hi) load_block(mine + NB * stride, ring[j]);
     }
   }
+  }
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) running_sum[ct] = groups_sum(running_sum[ct]);
 
-  if (waves > 1) {
+  if (!SHARED && waves > 1) {
     // ---- the waves' results into one, through LDS -------------------------------------------------
     extern __shared__ float lds[];
     float* stats = lds;                                  // [waves][CT][16][2]: maximum, sum
@@ -446,16 +570,16 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   }
 }
 
-template <int DT, int CT>
+template <int DT, int CT, bool SHARED = false>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
                             int split_len, int nq, int nkv, int page_size, int window, float scale, int waves,
                             hipStream_t stream) {
   const float scale_log2 = scale * 1.4426950408889634f;
   // LDS for merging the waves: their maxima and sums, and half as many slots as waves for the results
-  const size_t lds = waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
+  const size_t lds = !SHARED && waves > 1 ? (static_cast<size_t>(waves) * CT * 32 + static_cast<size_t>(waves / 2) * CT * DT * 256) * sizeof(float) : 0;
   if (lds > 64 * 1024) return kBadArgument;
-  hipLaunchKernelGGL((attention_mfma_kernel<DT, CT>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
+  hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                      (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
                      part_ml, nsplit, split_len, nq, nkv, page_size, window, scale_log2);
   return launch_status();
@@ -471,18 +595,25 @@ using namespace tlie;
 // part_o: float [tokens * nq * nsplit * d], part_ml: float [tokens * nq * nsplit * 2] (both only when nsplit > 1);
 // split_len: positions per part, a multiple of 32, nsplit * split_len >= the longest sequence.
 // d % 16 == 0, d <= 256, page_size a power of two >= 16; col_tiles 1, or 4 for d <= 64, or 2 for d <= 128.
+// shared != 0 (prompt portions, col_tiles 2, d <= 128, 4 or 8 waves): tiles have 32 * waves columns, every wave takes 32 of
+// them, and keys and values reach the waves through LDS.  Otherwise:
 // waves: 1, 2, 4 or 8 waves of a workgroup share a tile's keys; waves * col_tiles * d <= 1024 (their merge's LDS), and
 // at most 4 when col_tiles * d > 128.
 extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
                                    const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
                                    float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
-                                   int d, int page_size, int window, float scale, int waves, void* stream) {
+                                   int d, int page_size, int window, float scale, int waves, int shared, void* stream) {
   if (num_tiles <= 0 || tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || d % 16 != 0 ||
       page_size < 16 || (page_size & (page_size - 1)) != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
     return kBadArgument;
   if (nsplit > 1 && (part_o == nullptr || part_ml == nullptr || split_len <= 0 || split_len % 32 != 0)) return kBadArgument;
   if (col_tiles != 1 && !(col_tiles == 4 && d <= 64) && !(col_tiles == 2 && d <= 128)) return kBadArgument;
-  if (waves < 1 || (waves & (waves - 1)) != 0 || waves > attention_max_waves(d / 16, col_tiles)) return kBadArgument;
+  if (shared) {
+    // the waves take columns of their own: tiles of 16 * col_tiles * waves columns, 4 or 8 waves
+    if (tiles == nullptr || col_tiles != 2 || d > 128 || (waves != 4 && waves != 8)) return kBadArgument;
+  } else if (waves < 1 || (waves & (waves - 1)) != 0 || waves > attention_max_waves(d / 16, col_tiles)) {
+    return kBadArgument;
+  }
   if (tiles == nullptr && (col_tiles != 1 || num_tiles != tokens * ((nq / nkv + 15) / 16))) return kBadArgument;
   if (!(scale > 0.f)) return kBadArgument;     // the maximum is taken before the scores are scaled
   hipStream_t s = (hipStream_t)stream;
@@ -501,7 +632,15 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   case DT:                                                   \
     status = launch_attention<DT, 2>(TLIE_ARGS);             \
     break;
-  if (col_tiles == 1) {
+#define TLIE_SHARED(DT)                                      \
+  case DT:                                                   \
+    status = launch_attention<DT, 2, true>(TLIE_ARGS);       \
+    break;
+  if (shared) {
+    switch (d / 16) {
+      TLIE_SHARED(1) TLIE_SHARED(2) TLIE_SHARED(3) TLIE_SHARED(4) TLIE_SHARED(5) TLIE_SHARED(6) TLIE_SHARED(7) TLIE_SHARED(8)
+    }
+  } else if (col_tiles == 1) {
     switch (d / 16) {
       TLIE_CASE(1) TLIE_CASE(2) TLIE_CASE(3) TLIE_CASE(4) TLIE_CASE(5) TLIE_CASE(6) TLIE_CASE(7) TLIE_CASE(8)
       TLIE_CASE(9) TLIE_CASE(10) TLIE_CASE(11) TLIE_CASE(12) TLIE_CASE(13) TLIE_CASE(14) TLIE_CASE(15) TLIE_CASE(16)
@@ -514,6 +653,7 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
     }
   }
 #undef TLIE_CASE
+#undef TLIE_SHARED
 #undef TLIE_CASE2
 #undef TLIE_CASE4
 #undef TLIE_ARGS

@@ -83,20 +83,27 @@ class StepContext:
         as many parts as it takes to give a step of few tiles about a thousand waves (measured: at
         batch 64 and 2048 positions 4 parts reach 5 TB/s, 16 parts 4 TB/s, and merging more than 16
         costs more than it gains), each part a multiple of 32 positions and at least 64.
-        Returns (tiles, col_tiles, nsplit, split_len, waves of a workgroup that share a tile's keys)."""
+        Returns (tiles, col_tiles, nsplit, split_len, waves, shared): `waves` of a workgroup share a
+        tile's keys, or with `shared` take columns of their own and get the keys through LDS."""
         from ..ops import attention_max_waves
         decode = self.max_new == 1 and self.num_seqs == self.num_tokens
-        col_tiles = 1
+        col_tiles, shared = 1, False
         if decode:
             tiles, count = None, self.num_tokens * ((groups_per_kv + 15) // 16)
         else:
             from ..ops import attention_col_tiles, attention_tiles
             col_tiles = attention_col_tiles(head_dim)
-            if (groups_per_kv, col_tiles) not in self._tiles:
-                tiles = attention_tiles(self.host["seq_start"], groups_per_kv, col_tiles, self.host["seq_len"])
-                self._tiles[(groups_per_kv, col_tiles)] = torch.from_numpy(tiles).to(self.tokens.device)
-            tiles = self._tiles[(groups_per_kv, col_tiles)]
-            count = tiles.shape[0]
+            # long sequences with portions of many columns: 4 waves take 32 columns each of a tile
+            # of 128 and every block of keys is brought once for all of them, through LDS (a prompt
+            # of 2048 tokens: 80 us against 86; of 8192: 620 against 820; of 512: 18 against 15)
+            shared = (col_tiles == 2 and head_dim <= 128 and self.max_context >= 1536
+                      and self.num_tokens * groups_per_kv >= 128 * self.num_seqs)
+            groups = col_tiles * (4 if shared else 1)
+            if (groups_per_kv, groups) not in self._tiles:
+                tiles = attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"])
+                self._tiles[(groups_per_kv, groups)] = torch.from_numpy(tiles).to(self.tokens.device)
+            tiles = self._tiles[(groups_per_kv, groups)]
+            count = tiles.shape[0] * (4 if shared else 1)
         tiles_all = count * num_kv_heads
         if not decode:
             # a step of prompt portions has tiles enough; cutting their keys would only add merging.
@@ -104,8 +111,8 @@ class StepContext:
             # a long sequence then takes a quarter of the time, and it is the longest tiles that
             # the step waits for (a prompt of 2048 tokens: 70 us against 87 with one wave a tile)
             nsplit = max(1, min((512 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
-            waves = 1
-            while (waves < 4 and waves * 2 <= attention_max_waves(head_dim, col_tiles)
+            waves = 4 if shared else 1
+            while (not shared and waves < 4 and waves * 2 <= attention_max_waves(head_dim, col_tiles)
                    and self.max_context >= nsplit * waves * 2 * 128):
                 waves *= 2
         else:
@@ -120,10 +127,10 @@ class StepContext:
                    and self.max_context >= nsplit * waves * 2 * 128):
                 waves *= 2
         if nsplit == 1:
-            return tiles, col_tiles, 1, 0, waves
+            return tiles, col_tiles, 1, 0, waves, shared
         split_len = ((self.max_context + nsplit - 1) // nsplit + 31) // 32 * 32
         nsplit = (self.max_context + split_len - 1) // split_len
-        return tiles, col_tiles, nsplit, split_len, waves
+        return tiles, col_tiles, nsplit, split_len, waves, shared
 
 
 class ModelRunner:

@@ -394,7 +394,8 @@ def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> b
 
 def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor | None,
                    positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, window: int | None,
-                   scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1, waves: int = 1) -> torch.Tensor:
+                   scale: float, nsplit: int = 1, split_len: int = 0, col_tiles: int = 1, waves: int = 1,
+                   shared: bool = False) -> torch.Tensor:
     """Causal attention of every token of the step over its sequence's cache, bfloat16.
 
     tiles: int32 [n, 4] from `attention_tiles` (built from the same step as block_table and
@@ -403,7 +404,10 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     that many parts of split_len positions (a multiple of 32; nsplit * split_len must reach the
     longest sequence) that run side by side and are merged.  col_tiles: the value the tiles were
     made with.  waves (a power of two up to `attention_max_waves`): so many waves of a
-    workgroup share each tile's (or part's) keys and merge their results before writing."""
+    workgroup share each tile's (or part's) keys and merge their results before writing.
+    shared (prompt portions; col_tiles 2, head size up to 128, 4 or 8 waves): the tiles were made
+    with col_tiles * waves column groups, every wave takes col_tiles of them, and each block of keys
+    and values is brought once for the whole workgroup."""
     _device_tensor(q, "q", torch.bfloat16)
     _device_tensor(cache, "cache", torch.bfloat16)
     _device_tensor(block_table, "block_table", torch.int32)
@@ -432,7 +436,10 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
         num_tiles = tokens * ((num_heads // num_kv_heads + 15) // 16)
     if nsplit > 1 and (split_len <= 0 or split_len % 32 != 0):
         raise invalid_argument("attention: split_len must be a positive multiple of 32")
-    if waves not in (1, 2, 4, 8) or waves > attention_max_waves(head_dim, col_tiles):
+    if shared:
+        if tiles is None or col_tiles != 2 or head_dim > 128 or waves not in (4, 8):
+            raise invalid_argument("attention: sharing through LDS takes tiles, 2 column groups a wave, a head size up to 128 and 4 or 8 waves")
+    elif waves not in (1, 2, 4, 8) or waves > attention_max_waves(head_dim, col_tiles):
         raise invalid_argument(f"attention: waves must be a power of two up to {attention_max_waves(head_dim, col_tiles)}")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
         raise invalid_argument("attention_mfma takes bfloat16, head sizes in steps of 16 up to 256, pages of a power of two of rows (at least 16)")
@@ -444,7 +451,7 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     _check(library().tlie_attention_mfma(_ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[1], _ptr(tiles),
                                          num_tiles, col_tiles, _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), nsplit,
                                          split_len, tokens, num_heads, num_kv_heads, head_dim, page_size,
-                                         int(window) if window else 0, ctypes.c_float(scale), waves, _stream()),
+                                         int(window) if window else 0, ctypes.c_float(scale), waves, int(bool(shared)), _stream()),
            "attention_mfma")
     return out
 
