@@ -502,7 +502,7 @@ def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype):
         a.step(items)
         b.step(items)
         torch.cuda.synchronize()
-    assert 32 in recorded.runner._graphs and recorded.runner._graphs[32].graph is not None
+    assert (32, 256) in recorded.runner._graphs and recorded.runner._graphs[(32, 256)].graph is not None
     keys = sorted(a.rows, key=str)
     assert keys == sorted(b.rows, key=str)
     got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
@@ -529,7 +529,7 @@ def test_a_dropped_engine_frees_its_recordings_at_once(setups):
         engine.step([StepEntry("r", [1, 2, 3], [])])
         for token in (4, 5, 6):
             engine.step([StepEntry("r", [token], [0])])
-        recording = engine.runner._graphs[1]
+        recording = engine.runner._graphs[(1, 128)]
         assert recording.graph is not None
         watched = [weakref.ref(engine), weakref.ref(engine.runner), weakref.ref(recording), weakref.ref(recording.graph)]
         del recording
@@ -567,3 +567,25 @@ def test_long_prompts_take_the_walk_through_lds(tmp_path):
     policy = engine.runner.build_context([StepEntry("check", tokens[:1700], [])]).attention_tiles(2, 2, 16)
     assert policy[5] is True and policy[4] == 4
     engine.finish("check")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decoding_across_the_lengths_that_recordings_are_made_for(tmp_path, dtype):
+    """A recording of decode steps is made for sequences up to a power of two of positions (its
+    attention cuts the keys for that length).  A request that decodes from position 240 to 530
+    passes from the recording for 256 to the one for 512 and on to the one for the model's 600."""
+    raw = dict(CONFIGS["B"], max_position_embeddings=600, num_hidden_layers=1)
+    folder = make_model(tmp_path / "model", raw, seed=31, dtype_name=dtype)
+    stored, weights = load_plain(folder)
+    tokens = random_tokens(8, 531, raw["vocab_size"])
+    want = plain_forward(stored, weights, tokens)
+    from tlie_amd import Engine
+    engine = Engine(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=2)
+    replay = Replayer(engine)
+    replay.step([("r", tokens[:240], [239])])
+    for position in range(240, 531):
+        replay.step([("r", [tokens[position]], [0])])
+    engine.finish("r")
+    assert sorted(engine.runner._graphs) == [(1, 256), (1, 512), (1, 600)]
+    bad = first_bad_row(replay.logits_of("r", range(239, 531)), want[239:], TOLERANCE[dtype])
+    assert bad is None, f"first wrong position {239 + bad}"

@@ -144,7 +144,7 @@ class ModelRunner:
         # and replayed.  Parts say whether they may be captured (`graph_safe`).
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
         self.device_tokens: torch.Tensor | None = None     # int32, where sampling leaves a step's tokens (set by the engine)
-        self._graphs: dict[int, "DecodeGraph"] = {}
+        self._graphs: dict[tuple[int, int], "DecodeGraph"] = {}      # by (most sequences, longest sequence)
 
     # ---- checks and context ------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -175,6 +175,17 @@ class ModelRunner:
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
         return build_context(self.cache, entries, self.device, few_rows_dtype=self.model.dtype)
 
+    def _length_bucket(self, longest: int) -> int:
+        """The sequence length a recording is made for: the next power of two from 256 on, up to
+        what the cache can hold.  How attention cuts the keys is fixed in a recording, for its
+        longest sequence: one recording for the model's whole range would serve short sequences
+        of a long-range model with a handful of workgroups."""
+        limit = self.cache.max_positions or self.cache.num_pages * self.cache.page_size
+        bucket = 256
+        while bucket < longest:
+            bucket *= 2
+        return min(bucket, max(limit, longest))
+
     def replays(self, entries: Sequence[StepEntry]) -> bool:
         """Whether the step is one of single tokens, every logit wanted, that a recording serves."""
         return (self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH
@@ -198,10 +209,11 @@ class ModelRunner:
         if marks:
             marks[0].record()
         if self.replays(entries):
-            bucket = DecodeGraph.bucket_of(len(entries))
-            if bucket not in self._graphs:
-                self._graphs[bucket] = DecodeGraph(self, bucket)
-            logits = self._graphs[bucket].run(entries, marks[1] if marks else None)
+            longest = max(self.cache.length(request) + count for request, count in wanted)
+            key = (DecodeGraph.bucket_of(len(entries)), self._length_bucket(longest))
+            if key not in self._graphs:
+                self._graphs[key] = DecodeGraph(self, *key)
+            logits = self._graphs[key].run(entries, marks[1] if marks else None)
         else:
             if any(entry.source is not None for entry in entries):
                 raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
@@ -225,8 +237,9 @@ class DecodeGraph:
     the step's arrays live at fixed addresses, the model's kernels are recorded once into a HIP
     graph and replayed with new contents.  Rows beyond the step's sequences are padding: token 0
     at position 0 of a sequence with no page written (slot -1), whose results are dropped.
-    How the attention kernel cuts the key range is fixed at capture (for the longest sequence the
-    cache can hold); each part computes its own bounds from the positions on the device."""
+    How the attention kernel cuts the key range is fixed at capture, for sequences up to
+    `longest` positions (the runner keeps a recording per power of two); each part computes its own
+    bounds from the positions on the device."""
     MAX_BATCH = 64          # the largest step whose products all run in this engine's own kernels
 
     @staticmethod
@@ -236,7 +249,7 @@ class DecodeGraph:
             bucket *= 2
         return bucket
 
-    def __init__(self, runner: "ModelRunner", bucket: int):
+    def __init__(self, runner: "ModelRunner", bucket: int, longest: int):
         # The runner owns its recordings; a recording that owned its runner in turn would make the
         # pair garbage that only the cycle collector frees, at a moment of its choosing: if that
         # moment falls inside another recording's capture, the graph's destructor (which waits for
@@ -244,7 +257,7 @@ class DecodeGraph:
         self._runner = weakref.ref(runner)
         self.bucket = bucket
         cache = runner.cache
-        longest = cache.max_positions or cache.num_pages * cache.page_size
+        self.longest = longest
         self.widths = [max(1, (longest + cache.page_size - 1) // cache.page_size) for _ in cache.groups]
         layout = [("tokens", (bucket,)), ("positions", (bucket,)), ("token_seq", (bucket,)), ("no_slots", (bucket,)),
                   ("seq_start", (bucket + 1,)), ("seq_first_pos", (bucket,)), ("seq_len", (bucket,)), ("seq_slot", (bucket,)),
