@@ -65,6 +65,11 @@ __device__ __forceinline__ float groups_sum(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// The larger of two scores (no NaN, none above 3e38) as the median of them and 3e38: one
+// instruction, where fmaxf first makes sure that its operands are no signalling NaNs (an
+// instruction each for values that come from the matrix cores).
+__device__ __forceinline__ float larger(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, 3.0e38f); }
+
 // tiles[i] = (sequence row of the block table, index of the sequence's first token in this step,
 //             number of its tokens in this step, first column of the tile)
 // column c of a sequence = (token c / G of its tokens in this step, head c % G of the group).
@@ -133,8 +138,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   const int tile_hi = pos0 + last_col / G + 1;
   const int tile_lo = window > 0 ? max(0, pos0 + col0 / G - window + 1) : 0;
   const int split_lo = nsplit > 1 ? split * split_len : 0;
-  const int range_lo = wave_active ? max(tile_lo, split_lo) : 0;
-  const int range_hi = wave_active ? (nsplit > 1 ? min(tile_hi, split_lo + split_len) : tile_hi) : 0;
+  const int range_lo = __builtin_amdgcn_readfirstlane(wave_active ? max(tile_lo, split_lo) : 0);
+  const int range_hi = __builtin_amdgcn_readfirstlane(wave_active ? (nsplit > 1 ? min(tile_hi, split_lo + split_len) : tile_hi) : 0);
 
   // Pages hold a power of two of rows, at least 16, and blocks of 32 keys start at multiples of 32:
   // each half of a block (16 keys) lies on one page, the same for every lane.  So the page numbers
@@ -152,10 +157,10 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     table_high = pages[min(first_index + 64 + lane, max_blocks - 1)];
   };
   auto page_of = [&](int index) -> int {                   // index: the same for every lane, within the window
-    const int place = index - table_first;
+    const int place = __builtin_amdgcn_readfirstlane(index - table_first);
     const int low = __builtin_amdgcn_readlane(table_low, place & 63);
     const int high = __builtin_amdgcn_readlane(table_high, place & 63);
-    return place < 64 ? low : high;
+    return place < 64 ? low : high;                        // (all scalar: a select, not a mask)
   };
   const int table_span = 128 << page_shift;                // keys that one window covers
   const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * D;
@@ -250,65 +255,68 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
         for (int ks = 0; ks < KS; ++ks)
           s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(block.k[t][ks].v, qreg[ct][ks].v, s[ct][t], 0, 0, 0);
       }
-    // ---- mask and maximum (the scale goes into the exponent's multiply-add): s[ct][t][j] is key kb + t*16 + grp*4 + j of the column --------------
-    float block_max[CT];
+    // ---- mask; each lane's maximum over its 8 keys of a column (the scale goes into the exponent's
+    // multiply-add): s[ct][t][j] is key kb + t*16 + grp*4 + j of the column -------------------------
+    float lane_max[CT];
+    bool exceeds = false;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-      block_max[ct] = -INFINITY;
+      if (kMasked) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (kMasked) {
+          for (int j = 0; j < 4; ++j) {
             const int key = kb + t * 16 + grp * 4 + j;
             const bool ok = key >= range_lo && key < range_hi && key <= pos_col[ct] && key >= lo_col[ct];
             s[ct][t][j] = ok ? s[ct][t][j] : -INFINITY;
           }
-          block_max[ct] = fmaxf(block_max[ct], s[ct][t][j]);
-        }
+      }
+      lane_max[ct] = larger(larger(larger(s[ct][0][0], s[ct][0][1]), larger(s[ct][0][2], s[ct][0][3])),
+                            larger(larger(s[ct][1][0], s[ct][1][1]), larger(s[ct][1][2], s[ct][1][3]))) * scale_log2;   // the scale is positive
+      exceeds = exceeds || lane_max[ct] > running_max[ct];
     }
+    // ---- running softmax.  The running maximum of a column is shared by its four lane groups, and
+    // moves only when a block holds a larger score: rare once the first blocks have passed, so the
+    // reduction across the groups, and the rescaling of what has been summed so far, sit behind a
+    // branch of the whole wave.  Each group keeps the sum of its own keys; the groups' sums are
+    // added once, after the last block. ---------------------------------------------------------
+    if (__builtin_amdgcn_ballot_w64(exceeds) != 0) {
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) block_max[ct] = groups_max(block_max[ct]) * scale_log2;   // the scale is positive
-    // ---- running softmax: the column's four lane groups share the maximum, so each keeps the sum of
-    // its own keys and the groups' sums are added once, after the last block ------------------------
-    float alpha[CT];
+      for (int ct = 0; ct < CT; ++ct) {
+        const float new_max = fmaxf(running_max[ct], groups_max(lane_max[ct]));
+        const float alpha = new_max == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(running_max[ct] - new_max);   // 0 while the running maximum is -inf
+        running_max[ct] = new_max;
+        running_sum[ct] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) o[ct][dt][j] *= alpha;
+      }
+    }
     Pack8 p[CT];
-    bool changed = false;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
-      const float new_max = fmaxf(running_max[ct], block_max[ct]);
-      alpha[ct] = 1.f;
-      if (kMasked && new_max == -INFINITY) {
+      if (kMasked && running_max[ct] == -INFINITY) {
         p[ct].u = make_uint4(0, 0, 0, 0);              // nothing visible to this column yet
       } else {
-        alpha[ct] = __builtin_amdgcn_exp2f(running_max[ct] - new_max);      // 0 while the running maximum is -inf
         float e[8];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) e[t * 4 + j] = __builtin_amdgcn_exp2f(fmaf(s[ct][t][j], scale_log2, -new_max));   // 0 for masked keys
-        running_sum[ct] = running_sum[ct] * alpha[ct] + (((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7])));
+          for (int j = 0; j < 4; ++j) e[t * 4 + j] = __builtin_amdgcn_exp2f(fmaf(s[ct][t][j], scale_log2, -running_max[ct]));   // 0 for masked keys
+        running_sum[ct] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[ct].w[i] = pack_bf16(e[2 * i], e[2 * i + 1]);
       }
-      running_max[ct] = new_max;
-      changed = changed || alpha[ct] != 1.f;
     }
-    // ---- O^T = O^T * alpha + V^T . P^T -----------------------------------------------------------
-    const bool rescale = __builtin_amdgcn_ballot_w64(changed) != 0;      // rare once the maxima have settled
+    // ---- O^T += V^T . P^T -------------------------------------------------------------------------
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) {
       Pack8 a;
       a.h[0] = block.v[dt][0];
       a.h[1] = block.v[dt][1];
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct) {
-        if (rescale) {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) o[ct][dt][j] *= alpha[ct];
-        }
-        o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p[ct].v, o[ct][dt], 0, 0, 0);
-      }
+      for (int ct = 0; ct < CT; ++ct) o[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p[ct].v, o[ct][dt], 0, 0, 0);
     }
   };
 
@@ -324,8 +332,8 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   const int stride = 32 * waves;
   // a block that every column of the tile sees whole: inside the range, below the first column's
   // position, inside the last column's window
-  const int open_lo = max((range_lo + 31) & ~31, window > 0 ? tile_hi - window : 0);
-  const int open_hi = min(range_hi, pos0 + col0 / G + 1) & ~31;
+  const int open_lo = __builtin_amdgcn_readfirstlane(max((range_lo + 31) & ~31, window > 0 ? tile_hi - window : 0));
+  const int open_hi = __builtin_amdgcn_readfirstlane(min(range_hi, pos0 + col0 / G + 1) & ~31);
   auto work = [&](int kb, KeyBlock& block) {
     if (kb >= open_lo && kb + 32 <= open_hi)
       work_block(kb, block, std::false_type{});
@@ -353,21 +361,36 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
     constexpr int kAhead = DT <= 4 ? 4 : 2;                // (larger heads: the registers hold no more)
     typedef uint32_t Piece __attribute__((ext_vector_type(4)));     // a native vector: it stays in registers
     Piece staged_k[kAhead][kStage], staged_v[kAhead][kStage];
+    // where a thread's pieces lie within a half block's page rows: fixed for the whole walk, so that a
+    // block's addresses are two scalar bases (one per half, from its page numbers) plus these
+    int key_place[kStage], value_place[kStage];
+    bool key_second[kStage], value_second[kStage];
+#pragma unroll
+    for (int j = 0; j < kStage; ++j) {
+      // (threads beyond the block's pieces load the last piece again and do not store it: a load
+      // under a condition would hide from the compiler how many loads are on their way)
+      const int piece = min(static_cast<int>(threadIdx.x + j * blockDim.x), kPieces - 1);
+      const int key = piece / (D / 8), chunk = piece % (D / 8);
+      key_second[j] = key >= 16;
+      key_place[j] = (key & 15) * D + chunk * 8;
+      const int half = piece / (2 * D), rest = piece % (2 * D), dim = rest >> 1, part = rest & 1;
+      value_second[j] = half != 0;
+      value_place[j] = (dim << page_shift) + part * 8;
+    }
     auto bring = [&](int kb, Piece (&keys)[kStage], Piece (&values)[kStage]) {
-      const int page_a = page_of(kb >> page_shift);
-      const int page_b = page_of((kb + 16) >> page_shift);
+      // (a block starts at a multiple of 32 and a page holds at least 16 rows: each half's 16 keys are
+      // consecutive rows of one page)
+      const size_t page_a = static_cast<size_t>(page_of(kb >> page_shift)) * page_stride;
+      const size_t page_b = static_cast<size_t>(page_of((kb + 16) >> page_shift)) * page_stride;
+      const int row_a = kb & page_mask, row_b = (kb + 16) & page_mask;
+      const uint16_t* keys_a = k_base + page_a + row_a * D;
+      const uint16_t* keys_b = k_base + page_b + row_b * D;
+      const uint16_t* values_a = v_base + page_a + row_a;
+      const uint16_t* values_b = v_base + page_b + row_b;
 #pragma unroll
       for (int j = 0; j < kStage; ++j) {
-        // (threads beyond the block's pieces load the last piece again and do not store it: a load
-        // under a condition would hide from the compiler how many loads are on their way)
-        const int piece = min(static_cast<int>(threadIdx.x + j * blockDim.x), kPieces - 1);
-        const int key = piece / (D / 8), chunk = piece % (D / 8);
-        const size_t page = key < 16 ? page_a : page_b;
-        keys[j] = *reinterpret_cast<const Piece*>(k_base + page * page_stride + ((kb + key) & page_mask) * D + chunk * 8);
-        const int half = piece / (2 * D), rest = piece % (2 * D), dim = rest >> 1, part = rest & 1;
-        const size_t value_page = half == 0 ? page_a : page_b;
-        values[j] = *reinterpret_cast<const Piece*>(v_base + value_page * page_stride + (static_cast<size_t>(dim) << page_shift) +
-                                                    ((kb + half * 16) & page_mask) + part * 8);
+        keys[j] = *reinterpret_cast<const Piece*>((key_second[j] ? keys_b : keys_a) + key_place[j]);
+        values[j] = *reinterpret_cast<const Piece*>((value_second[j] ? values_b : values_a) + value_place[j]);
       }
     };
     auto put = [&](int buffer, const Piece (&keys)[kStage], const Piece (&values)[kStage]) {
