@@ -391,9 +391,10 @@ def test_attention_mfma(case):
             assert rel_err(shared, want) < TOL["bfloat16"], f"{waves} waves, {nsplit} parts"
     # the waves of a workgroup take columns of their own, keys and values reach them through LDS
     if d <= 128:
-        for waves, nsplit in ((4, 1), (8, 1), (4, 3)):
-            through_lds = run_attention_mfma(q, k, v, page, window, nsplit, shuffle_seed=tokens, col_tiles=2, waves=waves, shared=True)
-            assert rel_err(through_lds, want) < TOL["bfloat16"], f"through LDS, {waves} waves, {nsplit} parts"
+        for waves, nsplit, col_tiles in ((4, 1, 2), (8, 1, 2), (4, 3, 2), (4, 1, 1), (8, 2, 1)):
+            through_lds = run_attention_mfma(q, k, v, page, window, nsplit, shuffle_seed=tokens, col_tiles=col_tiles, waves=waves,
+                                             shared=True)
+            assert rel_err(through_lds, want) < TOL["bfloat16"], f"through LDS, {waves} waves of {col_tiles * 16} columns, {nsplit} parts"
     # the last token alone (a decode step), its key range cut in parts that are merged
     for nsplit in (1, 2, 5):
         last = run_attention_mfma(q, k, v, page, window, nsplit, token_list=[tokens - 1], shuffle_seed=tokens)
@@ -406,6 +407,9 @@ def test_attention_mfma(case):
         portion = run_attention_mfma(q, k, v, page, window, 1, token_list=list(range(first, first + count)), shuffle_seed=tokens,
                                      col_tiles=2, waves=4, shared=True)
         assert rel_err(portion, want[first:first + count]) < TOL["bfloat16"], "a portion through LDS"
+        portion = run_attention_mfma(q, k, v, page, window, 1, token_list=list(range(first, first + count)), shuffle_seed=tokens,
+                                     col_tiles=1, waves=4, shared=True)
+        assert rel_err(portion, want[first:first + count]) < TOL["bfloat16"], "a portion through LDS, 16 columns a wave"
     split_portion = run_attention_mfma(q, k, v, page, window, 3, token_list=list(range(first, first + count)), shuffle_seed=tokens)
     assert rel_err(split_portion, want[first:first + count]) < TOL["bfloat16"]
 

@@ -95,18 +95,32 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nsplit, int split_len, int nq, int nkv, int page_size,
-                      int window, float scale_log2) {
+                      int window, float scale_log2, int round_size) {
   constexpr int D = DT * 16;
   constexpr int KS = (DT + 1) / 2;                 // 32-wide k steps of the first product
   const int lane = threadIdx.x & 63, col = lane & 15, grp = lane >> 4;
   const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;     // waves that share the tile's keys
-  const int kvh = blockIdx.y, split = blockIdx.z;
+  // Which (tile, kv head) this workgroup takes.  The tiles come sorted, longest first, and all kv
+  // heads of a tile are equally long.  Workgroups start in the order of their index, one round of
+  // round_size (the number of CUs) after the other; the rounds run through the sorted list forwards
+  // and backwards in turn, so that a CU that got a long tile in one round gets a short one in the
+  // next: when the whole grid is resident at once (a prompt of a few thousand tokens) the CUs then
+  // finish together, where equal partners would leave half of them idle half of the time.
+  int tile_index = blockIdx.x, kvh = blockIdx.y;
+  if (tiles != nullptr && round_size > 0) {
+    const int total = gridDim.x * gridDim.y, linear = blockIdx.y * gridDim.x + blockIdx.x;
+    const int round = linear / round_size, place = linear - round * round_size;
+    const int in_round = min(round_size, total - round * round_size);
+    const int item = round * round_size + ((round & 1) ? in_round - 1 - place : place);
+    tile_index = item / static_cast<int>(gridDim.y), kvh = item - tile_index * static_cast<int>(gridDim.y);
+  }
+  const int split = blockIdx.z;
   // whether a lane's 8 dims of k step ks exist: always, unless the head size is an odd multiple of 16
   auto has_dims = [&](int ks) { return DT % 2 == 0 || ks < KS - 1 || grp < 2; };
   const int G = nq / nkv;
   int seq, tok0, ntok, col0;
   if (tiles != nullptr) {
-    const int4 tile = tiles[blockIdx.x];
+    const int4 tile = tiles[tile_index];
     seq = tile.x, tok0 = tile.y, ntok = tile.z, col0 = tile.w;
   } else {
     const int per_seq = (G + 16 * CT - 1) / (16 * CT);
@@ -593,6 +607,19 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   }
 }
 
+// the number of CUs of the current device (asked once per device)
+static int compute_units() {
+  static int cached[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+  if (cached[device] == 0) {
+    int count = 0;
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess) return 0;
+    cached[device] = count;
+  }
+  return cached[device];
+}
+
 template <int DT, int CT, bool SHARED = false>
 static int launch_attention(const void* q, const void* cache, const int* block_table, int max_blocks, const void* tiles,
                             int num_tiles, const int* positions, void* out, float* part_o, float* part_ml, int nsplit,
@@ -604,7 +631,7 @@ static int launch_attention(const void* q, const void* cache, const int* block_t
   if (lds > 64 * 1024) return kBadArgument;
   hipLaunchKernelGGL((attention_mfma_kernel<DT, CT, SHARED>), dim3(num_tiles, nkv, nsplit), dim3(64 * waves), lds, stream, (const uint16_t*)q,
                      (const uint16_t*)cache, block_table, max_blocks, (const int4*)tiles, positions, (uint16_t*)out, part_o,
-                     part_ml, nsplit, split_len, nq, nkv, page_size, window, scale_log2);
+                     part_ml, nsplit, split_len, nq, nkv, page_size, window, scale_log2, compute_units());
   return launch_status();
 }
 
@@ -618,8 +645,8 @@ using namespace tlie;
 // part_o: float [tokens * nq * nsplit * d], part_ml: float [tokens * nq * nsplit * 2] (both only when nsplit > 1);
 // split_len: positions per part, a multiple of 32, nsplit * split_len >= the longest sequence.
 // d % 16 == 0, d <= 256, page_size a power of two >= 16; col_tiles 1, or 4 for d <= 64, or 2 for d <= 128.
-// shared != 0 (prompt portions, col_tiles 2, d <= 128, 4 or 8 waves): tiles have 32 * waves columns, every wave takes 32 of
-// them, and keys and values reach the waves through LDS.  Otherwise:
+// shared != 0 (prompt portions, col_tiles 1 or 2, d <= 128, 4 or 8 waves): tiles have 16 * col_tiles * waves columns, every wave
+// takes 16 * col_tiles of them, and keys and values reach the waves through LDS.  Otherwise:
 // waves: 1, 2, 4 or 8 waves of a workgroup share a tile's keys; waves * col_tiles * d <= 1024 (their merge's LDS), and
 // at most 4 when col_tiles * d > 128.
 extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
@@ -633,7 +660,7 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   if (col_tiles != 1 && !(col_tiles == 4 && d <= 64) && !(col_tiles == 2 && d <= 128)) return kBadArgument;
   if (shared) {
     // the waves take columns of their own: tiles of 16 * col_tiles * waves columns, 4 or 8 waves
-    if (tiles == nullptr || col_tiles != 2 || d > 128 || (waves != 4 && waves != 8)) return kBadArgument;
+    if (tiles == nullptr || (col_tiles != 2 && col_tiles != 1) || d > 128 || (waves != 4 && waves != 8)) return kBadArgument;
   } else if (waves < 1 || (waves & (waves - 1)) != 0 || waves > attention_max_waves(d / 16, col_tiles)) {
     return kBadArgument;
   }
@@ -655,9 +682,10 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   case DT:                                                   \
     status = launch_attention<DT, 2>(TLIE_ARGS);             \
     break;
-#define TLIE_SHARED(DT)                                      \
-  case DT:                                                   \
-    status = launch_attention<DT, 2, true>(TLIE_ARGS);       \
+#define TLIE_SHARED(DT)                                                              \
+  case DT:                                                                           \
+    status = col_tiles == 2 ? launch_attention<DT, 2, true>(TLIE_ARGS)               \
+                            : launch_attention<DT, 1, true>(TLIE_ARGS);              \
     break;
   if (shared) {
     switch (d / 16) {

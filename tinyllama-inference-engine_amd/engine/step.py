@@ -75,6 +75,7 @@ class StepContext:
     host: dict                     # the same arrays as numpy, by name
     few_rows: bool = False         # at most 16 tokens of bfloat16: the step may use the products that fold norms and adds in
     wants_all_rows: bool = False   # the wanted rows are all the step's tokens, in order
+    compute_units: int = 256       # of the device: how many workgroups start at once
     _tiles: dict = field(default_factory=dict)
 
     def attention_tiles(self, groups_per_kv: int, num_kv_heads: int, head_dim: int):
@@ -93,16 +94,24 @@ class StepContext:
         else:
             from ..ops import attention_col_tiles, attention_tiles
             col_tiles = attention_col_tiles(head_dim)
-            # long sequences with portions of many columns: 4 waves take 32 columns each of a tile
-            # of 128 and every block of keys is brought once for all of them, through LDS (a prompt
-            # of 2048 tokens: 80 us against 86; of 8192: 620 against 820; of 512: 18 against 15)
-            shared = (col_tiles == 2 and head_dim <= 128 and self.max_context >= 1536
-                      and self.num_tokens * groups_per_kv >= 128 * self.num_seqs)
-            groups = col_tiles * (4 if shared else 1)
-            if (groups_per_kv, groups) not in self._tiles:
-                tiles = attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"])
-                self._tiles[(groups_per_kv, groups)] = torch.from_numpy(tiles).to(self.tokens.device)
-            tiles = self._tiles[(groups_per_kv, groups)]
+            # sequences of some length with portions of many columns: 4 waves take columns of their own
+            # of one tile and every block of keys is brought once for all of them, through LDS (a
+            # prompt of 1536 tokens: 34 us against 42; of 8192: 500 against 780; of 512: 15 against
+            # 13).  Each wave takes 32 columns, or 16 while that leaves no more tiles than two for
+            # every compute unit: they are then all at work at once, and smaller ones fill the chip
+            # better (1024 tokens: 24 us against 30; from 3072 on the larger tiles win)
+            shared = (col_tiles == 2 and head_dim <= 128 and self.max_context >= 768
+                      and self.num_tokens * groups_per_kv >= 64 * self.num_seqs)
+
+            def tiles_of(groups):
+                if (groups_per_kv, groups) not in self._tiles:
+                    made = attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"])
+                    self._tiles[(groups_per_kv, groups)] = torch.from_numpy(made).to(self.tokens.device)
+                return self._tiles[(groups_per_kv, groups)]
+            tiles = tiles_of(col_tiles * (4 if shared else 1))
+            if shared and tiles.shape[0] * num_kv_heads <= 2 * self.compute_units:
+                col_tiles = 1
+                tiles = tiles_of(4)
             count = tiles.shape[0] * (4 if shared else 1)
         tiles_all = count * num_kv_heads
         if not decode:
@@ -386,6 +395,13 @@ class DecodeGraph:
         return self.logits[:len(entries)]
 
 
+def _compute_units(device) -> int:
+    device = torch.device(device)
+    if device.type != "cuda":
+        return 256
+    return int(torch.cuda.get_device_properties(device).multi_processor_count)
+
+
 def build_context(cache: CacheManager, entries: Sequence[StepEntry], device, few_rows_dtype=None) -> StepContext:
     """The step's arrays for entries whose pages are reserved: built on the host, sent in one
     transfer."""
@@ -437,5 +453,6 @@ def build_context(cache: CacheManager, entries: Sequence[StepEntry], device, few
         seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
         want_rows=views["want_rows"], groups=groups, host=host,
         few_rows=total <= 16 and few_rows_dtype == torch.bfloat16,
-        wants_all_rows=bool(want_rows.size == total and np.array_equal(want_rows, np.arange(total))))
+        wants_all_rows=bool(want_rows.size == total and np.array_equal(want_rows, np.arange(total))),
+        compute_units=_compute_units(device))
 

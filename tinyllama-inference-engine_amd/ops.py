@@ -405,7 +405,7 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     longest sequence) that run side by side and are merged.  col_tiles: the value the tiles were
     made with.  waves (a power of two up to `attention_max_waves`): so many waves of a
     workgroup share each tile's (or part's) keys and merge their results before writing.
-    shared (prompt portions; col_tiles 2, head size up to 128, 4 or 8 waves): the tiles were made
+    shared (prompt portions; col_tiles 1 or 2, head size up to 128, 4 or 8 waves): the tiles were made
     with col_tiles * waves column groups, every wave takes col_tiles of them, and each block of keys
     and values is brought once for the whole workgroup."""
     _device_tensor(q, "q", torch.bfloat16)
@@ -437,8 +437,8 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
     if nsplit > 1 and (split_len <= 0 or split_len % 32 != 0):
         raise invalid_argument("attention: split_len must be a positive multiple of 32")
     if shared:
-        if tiles is None or col_tiles != 2 or head_dim > 128 or waves not in (4, 8):
-            raise invalid_argument("attention: sharing through LDS takes tiles, 2 column groups a wave, a head size up to 128 and 4 or 8 waves")
+        if tiles is None or col_tiles not in (1, 2) or head_dim > 128 or waves not in (4, 8):
+            raise invalid_argument("attention: sharing through LDS takes tiles, 1 or 2 column groups a wave, a head size up to 128 and 4 or 8 waves")
     elif waves not in (1, 2, 4, 8) or waves > attention_max_waves(head_dim, col_tiles):
         raise invalid_argument(f"attention: waves must be a power of two up to {attention_max_waves(head_dim, col_tiles)}")
     if not attention_mfma_takes(q.dtype, head_dim, page_size):
