@@ -337,7 +337,10 @@ def run_attention_mfma(q, k, v, page, window, nsplit, token_list=None, shuffle_s
     tiles = ops.attention_tiles(np.asarray([0, len(token_list)]), nq // nkv, col_tiles * (waves if shared else 1),
                                 np.asarray([token_list[-1] + 1]) if waves > 1 else None)
     if waves > 1 and tiles.shape[0] > 1:
-        assert tiles[0, 3] > tiles[-1, 3]                                      # the tile of the last tokens first
+        # the tiles that see the most keys come first (a tile's last column decides)
+        groups, columns = col_tiles * (waves if shared else 1), len(token_list) * (nq // nkv)
+        reach = [(min(int(col0) + 16 * groups, columns) - 1) // (nq // nkv) for col0 in tiles[:, 3]]
+        assert reach == sorted(reach, reverse=True)
     tiles[:, 0] = 1                                                            # the sequence is row 1 of the table
     split_len = ((tokens + nsplit - 1) // nsplit + 31) // 32 * 32
     rows = q[token_list].bfloat16().reshape(len(token_list), nq * d).contiguous().to(DEV)
