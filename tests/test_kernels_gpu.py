@@ -437,6 +437,30 @@ def test_attention_mfma_finds_one_key_among_hundreds():
             assert hit == inside, f"window {window}, needle at {needle}, nsplit {nsplit}: {'missed' if inside else 'seen'}"
 
 
+def test_attention_mfma_over_thousands_of_keys():
+    """A sequence of more pages than the 128 whose numbers a wave keeps at hand while it brings
+    blocks through LDS (2600 positions in pages of 16): the last tokens' queries against all keys, by
+    every walk, and needles on both sides of the place where the page numbers are loaded again."""
+    tokens, nq, nkv, d, page = 2600, 4, 2, 32, 16
+    torch.manual_seed(5)
+    k, v = torch.randn(tokens, nkv, d) * 0.1, torch.randn(tokens, nkv, d)
+    q = torch.randn(tokens, nq, d) * 0.1
+    direction = torch.zeros(d)
+    direction[5] = 1.0
+    first, count = tokens - 150, 150
+    for needle in (0, 2047, 2048, 2080, tokens - 151):
+        keys = k.clone()
+        keys[needle] += 12.0 * direction
+        queries = q.clone()
+        queries[first:] += 12.0 * direction
+        want = plain_attention(rounded(queries, torch.bfloat16), rounded(keys, torch.bfloat16), rounded(v, torch.bfloat16))[first:]
+        assert (want - v[needle].bfloat16().double().repeat_interleave(nq // nkv, dim=0)).abs().max() < 0.05   # the needle decides
+        for col_tiles, waves, shared, nsplit in ((2, 4, True, 1), (1, 4, True, 1), (2, 8, True, 2), (2, 4, False, 1), (1, 1, False, 3)):
+            got = run_attention_mfma(queries, keys, v, page, None, nsplit, token_list=list(range(first, first + count)),
+                                     shuffle_seed=needle, col_tiles=col_tiles, waves=waves, shared=shared)
+            assert rel_err(got, want) < TOL["bfloat16"], f"needle {needle}: {col_tiles} groups, {waves} waves, shared {shared}, {nsplit} parts"
+
+
 def test_attention_mfma_mixed_step():
     """Three sequences in one step: a portion of a prompt, one decoded token, a whole short prompt;
     each must equal what it gives alone."""
