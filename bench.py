@@ -1,6 +1,7 @@
 """Measures decoding and prefill of the TinyLlama 1.1B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--dtype bfloat16]
+                    [--shape tinyllama|llama2_7b|llama3_8b] [--layers N] [--no-points]
 
 A step is one decode step of the whole batch.  The batch's requests are first prefilled so that
 after the warm-up and the K timed steps their length is `context`; then W untimed and exactly K
@@ -27,6 +28,15 @@ TINYLLAMA = dict(model_type="llama", architectures=["LlamaForCausalLM"], hidden_
                  num_hidden_layers=22, num_attention_heads=32, num_key_value_heads=4, max_position_embeddings=2048,
                  vocab_size=32000, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False, attention_bias=False,
                  hidden_act="silu", bos_token_id=1, eos_token_id=2, torch_dtype="bfloat16")
+
+
+# the layer sizes of BASELINE.json's configs[3] and configs[4], for `--shape`
+OTHER_SHAPES = {
+    "llama2_7b": ("Llama-2-7B shape", dict(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
+                                           num_key_value_heads=32, max_position_embeddings=4096, vocab_size=32000, rope_theta=10000.0)),
+    "llama3_8b": ("Llama-3-8B shape", dict(hidden_size=4096, intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32,
+                                           num_key_value_heads=8, max_position_embeddings=8192, vocab_size=128256, rope_theta=500000.0)),
+}
 
 
 def weight_bytes_per_step(cfg, itemsize):
@@ -108,13 +118,18 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the configuration has (named in the record)")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],
+                        help="layer sizes of another model of the same architecture (the default is the record's)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on a single MI355X)")
         return 2
     import torch
     from tlie_amd import Engine
-    cfg = dict(TINYLLAMA)
+    cfg, model_name = dict(TINYLLAMA), "TinyLlama 1.1B shape"
+    if args.shape != "tinyllama":
+        model_name = OTHER_SHAPES[args.shape][0]
+        cfg.update(OTHER_SHAPES[args.shape][1])
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -134,11 +149,11 @@ def main() -> int:
     step_bytes = weight_bytes_per_step(cfg, itemsize) + args.batch * mean_context * kv_bytes_per_token(cfg, itemsize)
     achieved = step_bytes / (elapsed / args.steps)
     record = {
-        "metric": f"decode tok/s at batch {args.batch}, context {args.context} (TinyLlama 1.1B shape)", "value": value, "unit": "tokens/s",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({model_name})", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
-        "config": {"model": "TinyLlama-1.1B shape", "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
+        "config": {"model": model_name, "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "ffn": cfg["intermediate_size"],
                    "vocab": vocab, "global_batch": args.batch, "seq_len": args.context, "page_size": 16,
