@@ -76,7 +76,8 @@ __device__ __forceinline__ float larger(float a, float b) { return __builtin_amd
 // tiles == nullptr: a decode step, token i is the one token of sequence i; the tile index is
 // sequence * ceil(G / 16) + tile of the group.
 // DT = head_dim / 16.  CT = groups of 16 columns per wave: a tile has 16 * CT columns, and every
-// key and value the wave loads serves all of them (prompt portions take CT = 4, decode steps 1).
+// key and value the wave loads serves all of them (prompt portions take CT = 1 or 2, decode steps 1;
+// 4 fit the registers for head sizes up to 64 and measured slower).
 // A workgroup has at most 8 waves, and at most 1024 / (16 * CT * DT): their merge fits LDS, and
 // every wave may use 256 registers;
 // head sizes above 128 need more registers still and get 4 waves at most.

@@ -149,8 +149,8 @@ class ModelRunner:
         self.device = model.device
         self.vocab_size = model.spec.vocab_size
         # Decode steps are bound by launches, not by the kernels: a step of single tokens whose
-        # kernels are all this engine's own is captured once per batch-size bucket as a HIP graph
-        # and replayed.  Parts say whether they may be captured (`graph_safe`).
+        # kernels are all this engine's own is captured once per batch-size bucket and range of
+        # sequence lengths as a HIP graph and replayed.  Parts say whether they may be captured (`graph_safe`).
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
         self.device_tokens: torch.Tensor | None = None     # int32, where sampling leaves a step's tokens (set by the engine)
         self._graphs: dict[tuple[int, int], "DecodeGraph"] = {}      # by (most sequences, longest sequence)
