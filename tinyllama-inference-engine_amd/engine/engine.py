@@ -187,7 +187,6 @@ class Engine:
             else:
                 return None
         if any(source is not None for source in sources):
-            probe = [StepEntry(item.request.id, [0] * item.count, [item.count - 1] if item.samples else []) for item in plan]
-            if not self.runner.replays(probe):
+            if not (all(item.count == 1 and item.samples for item in plan) and self.runner.replays_single_tokens(len(plan))):
                 return None
         return sources

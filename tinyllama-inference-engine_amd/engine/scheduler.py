@@ -166,15 +166,20 @@ class Scheduler:
         plan: list[Scheduled] = []
         planned_pages = [0] * len(self.cache.groups)
 
-        def fits(request: Request, count: int) -> bool:
-            needed = self.cache.pages_needed(request.id, count)
-            return all(planned + need <= free for planned, need, free in zip(planned_pages, needed, self.cache.free_pages()))
+        planned: set = set()                 # ids of the requests that the plan holds
 
-        def take(request: Request, count: int) -> None:
+        def needs(request: Request, count: int) -> list[int]:
+            return self.cache.pages_needed(request.id, count)
+
+        def fits(needed: list[int]) -> bool:
+            return all(held + need <= free for held, need, free in zip(planned_pages, needed, self.cache.free_pages()))
+
+        def take(request: Request, count: int, needed: list[int] | None = None) -> None:
             nonlocal budget
-            for group, need in enumerate(self.cache.pages_needed(request.id, count)):
+            for group, need in enumerate(needed if needed is not None else needs(request, count)):
                 planned_pages[group] += need
             plan.append(Scheduled(request, request.computed, count, request.computed + count == request.total))
+            planned.add(request.id)
             budget -= count
 
         # 1. requests that decode: one token each, from the cursor when they exceed the budget
@@ -185,19 +190,23 @@ class Scheduler:
             decoding = (decoding[start:] + decoding[:start])[:limit]
             self._cursor += limit
         for request in decoding:
-            while request.state == "running" and not fits(request, 1):
+            if request.state != "running":             # preempted for a request before it in this loop
+                continue
+            needed = needs(request, 1)
+            while request.state == "running" and not fits(needed):
                 victim = max(self.running, key=lambda candidate: candidate.order)
                 if victim is request and len(self.running) == 1:
                     raise out_of_memory(f"request {request.id!r} does not fit the pool alone")   # add() rules this out
                 self._preempt(victim, plan, planned_pages)
+                planned.discard(victim.id)
             if request.state == "running":
-                take(request, 1)
+                take(request, 1, needed)
 
         # 2. running requests still in their prompt (or being recomputed), in admission order
         for request in sorted(self.running, key=lambda candidate: candidate.order):
             if budget <= 0 or len(plan) >= self.max_seqs_per_step:
                 break
-            if any(item.request is request for item in plan) or request.remaining == 0:
+            if request.id in planned or request.remaining == 0:
                 continue
             count = self._portion(request, budget, planned_pages)
             if count > 0:

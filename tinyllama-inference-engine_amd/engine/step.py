@@ -195,9 +195,13 @@ class ModelRunner:
             bucket *= 2
         return min(bucket, max(limit, longest))
 
+    def replays_single_tokens(self, count: int) -> bool:
+        """Whether a recording serves a step of `count` entries of one token each, every logit wanted."""
+        return self.use_graphs and count <= DecodeGraph.MAX_BATCH
+
     def replays(self, entries: Sequence[StepEntry]) -> bool:
         """Whether the step is one of single tokens, every logit wanted, that a recording serves."""
-        return (self.use_graphs and len(entries) <= DecodeGraph.MAX_BATCH
+        return (self.replays_single_tokens(len(entries))
                 and all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries))
 
     # ---- the step ----------------------------------------------------------------------------
