@@ -34,7 +34,10 @@ def _ptr(tensor: torch.Tensor | None):
 
 
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the current stream of the current device, by the accessors that cost no Python (a step of
+    # prompt portions makes some two hundred launches, and torch.cuda.current_stream() alone took
+    # a quarter of the time the host needs for them)
+    return ctypes.c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def _check(status: int, what: str) -> None:
