@@ -102,6 +102,22 @@ def test_gemm_generic(dtype, shape):
     assert rel_err(got, plain_linear(x.double(), w.double())) < TOL[dtype]
 
 
+@pytest.mark.parametrize("shape", [(3, 50, 37), (16, 129, 640), (17, 33, 131), (64, 200, 2052), (9, 2048, 5632)])
+def test_gemm_generic_gives_few_rows_the_same_bits_as_many(shape):
+    """Few rows take a kernel of their own; a row's sums must not depend on which one ran: the
+    first rows of a batch of 100 against the same rows alone, bit for bit."""
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(k)
+    x = torch.randn(100, k, device=DEV)
+    w = torch.randn(n, k, device=DEV) / math.sqrt(k)
+    b = torch.randn(n, device=DEV)
+    many = ops.gemm_generic(x, w, b, torch.float32).dense()
+    few = ops.gemm_generic(x[:m].contiguous(), w, b, torch.float32).dense()
+    assert torch.equal(few, many[:m])
+    assert rel_err(few, plain_linear(x[:m].double().cpu(), w.double().cpu(), b.double().cpu())) < 5e-6
+
+
 def test_gemm_is_true_32_bit():
     """(1 + 2^-12)^2 accumulated onto -(1 + 2^-11) leaves 2^-24: it needs all 24 bits of both
     factors and a fused multiply-add; a product whose inputs were cut to fewer bits leaves -2^-11
