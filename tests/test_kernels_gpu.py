@@ -118,6 +118,22 @@ def test_gemm_generic_gives_few_rows_the_same_bits_as_many(shape):
     assert rel_err(few, plain_linear(x[:m].double().cpu(), w.double().cpu(), b.double().cpu())) < 5e-6
 
 
+@pytest.mark.parametrize("shape", [(65, 96, 64), (200, 2560, 2048), (333, 177, 200), (70, 129, 333), (1024, 2048, 5632)])
+def test_library_product_of_many_rows(shape):
+    """The vendor library's product, called directly where it offers an algorithm (and through
+    torch where it does not: odd inner sizes), against the plain product of the rounded inputs."""
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(n)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    got = ops.library_mm(x.to(DEV), w.to(DEV))
+    assert got.dtype == torch.bfloat16 and got.shape == (m, n)
+    assert rel_err(got, plain_linear(x.double(), w.double())) < TOL["bfloat16"]
+    again = ops.library_mm(x.to(DEV), w.to(DEV))              # the kept plan
+    assert torch.equal(got, again)
+
+
 def test_gemm_is_true_32_bit():
     """(1 + 2^-12)^2 accumulated onto -(1 + 2^-11) leaves 2^-24: it needs all 24 bits of both
     factors and a fused multiply-add; a product whose inputs were cut to fewer bits leaves -2^-11

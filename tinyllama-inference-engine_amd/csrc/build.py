@@ -16,7 +16,7 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["elementwise.hip", "rope_cache.hip", "attention_generic.hip", "attention_mfma.hip", "gemm_generic.hip",
-           "gemm_skinny.hip", "gemm_rows.hip", "sampling.hip"]
+           "gemm_skinny.hip", "gemm_rows.hip", "sampling.hip", "library_gemm.hip"]
 HEADERS = ["common.h"]
 LIBRARY = "libtlie_hip.so"
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",
@@ -88,7 +88,7 @@ def build(verbose: bool = True) -> str:
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {name}:\n{output}")
     temporary = path + f".tmp{os.getpid()}"
-    link = subprocess.run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", temporary],
+    link = subprocess.run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-ldl", "-o", temporary],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if link.returncode != 0:
         raise RuntimeError(f"hipcc failed to link {LIBRARY}:\n{link.stdout}")

@@ -265,6 +265,41 @@ def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | Non
     return Product(out, 1)
 
 
+_library_gemm = {"state": None, "workspace": {}}       # state: None (not tried), True, False (not there)
+LIBRARY_WORKSPACE_BYTES = 32 << 20
+
+
+def library_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """y = x . W^T in bfloat16 through the vendor's library (hipBLASLt), for steps of many rows.
+    The library is called directly, with its plan for the shape kept (half the host time of
+    torch.mm, which a step of prompt portions calls four times a layer); where that is not
+    possible (the library's file is not beside torch, or it has no algorithm for the shape)
+    torch.mm makes the same product."""
+    _device_tensor(x, "x", torch.bfloat16)
+    _device_tensor(weight, "weight", torch.bfloat16)
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise invalid_shape(f"library_mm: x {list(x.shape)} and weight {list(weight.shape)} do not fit")
+    state = _library_gemm
+    if state["state"] is None:
+        import os
+        path = os.path.join(os.path.dirname(torch.__file__), "lib", "libhipblaslt.so")
+        torch.mm(x[:1], weight[:1].t())                       # torch loads and sets up its copy of the library first
+        state["state"] = os.path.isfile(path) and library().tlie_library_gemm_init(path.encode()) == 0
+    if state["state"] and x.shape[0] > 0:
+        index = x.device.index or 0
+        if index not in state["workspace"]:
+            state["workspace"][index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
+        workspace = state["workspace"][index]
+        out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.bfloat16, device=x.device)
+        status = library().tlie_library_gemm(_ptr(x), _ptr(weight), _ptr(out), x.shape[0], weight.shape[0], x.shape[1],
+                                             _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
+        if status == 0:
+            return out
+        if status != -3:
+            _check(status, "library_gemm")
+    return torch.mm(x, weight.t())
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
            seed: torch.Tensor | None = None, counter: torch.Tensor | None = None,
            out: torch.Tensor | None = None) -> torch.Tensor:

@@ -8,7 +8,8 @@ Which kernel runs is decided here and nowhere else:
                                  product, the SiLU gate or the add into the residual after it
   bfloat16, at most 64 rows      the skinny MFMA kernel (W streamed once, split-K partial sums)
   bfloat16, more rows            the library's product (as the reference uses a library for its
-                                 products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out
+                                 products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out:
+                                 hipBLASLt called directly (`ops.library_mm`), torch.mm where that fails
   anything those refuse          the plain kernel
 """
 from __future__ import annotations
@@ -65,5 +66,5 @@ class Linear:
                 raise ops.invalid_shape(f"linear: x {list(x.shape)} does not fit weight {list(self.weight.shape)}")
             if self.bias is not None:
                 return Product(torch.addmm(self.bias, x, self.weight.t()), 1)
-            return Product(torch.mm(x, self.weight.t()), 1)
+            return Product(ops.library_mm(x, self.weight), 1)
         return ops.gemm_generic(x, self.weight, self.bias, out_dtype)
