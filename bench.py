@@ -171,6 +171,8 @@ def main() -> int:
             steps = min(args.steps, 64)
             seconds = time_decode(engine, torch, batch, args.context, steps, 4, vocab)
             points[f"decode_b{batch}"] = batch * steps / seconds
+        # a short prompt: its step is replayed from a recording (the long one's is launched kernel by kernel)
+        points["prefill_256"] = 256 / time_prefill(engine, torch, 256, vocab)
         record["points"] = points
     print(json.dumps(record))
     return 0

@@ -209,6 +209,56 @@ def test_greedy_generation_through_the_entry_point(setups, name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
+def test_recorded_portion_steps_replay_like_eager_ones(setups, name, dtype):
+    """Steps of prompt portions (beside single tokens) of up to some hundred tokens are recorded
+    too, per (tokens, sequences, longest sequence) padded up, with the attention kernel's work list
+    at a fixed size.  The same recording is replayed with the step cut in other ways each time
+    (other portions, other sequences, fewer tokens than it holds, pages in another order), with
+    eager steps (all rows wanted: never recorded) and synchronisations in between, and every
+    replay is checked against an engine that launches one kernel at a time."""
+    setup = setups(name, dtype)
+    recorded, eager = new_engine(setup, dtype, max_tokens=1024, max_requests=8), \
+        new_engine(setup, dtype, max_tokens=1024, max_requests=8, use_graphs=False)
+    rng = random.Random(5)
+    streams = {f"p{i}": request_tokens(name, 40 + i, n) for i, n in enumerate((97, 64, 31, 120))}
+    done = {request: 0 for request in streams}
+    a, b = Replayer(recorded), Replayer(eager)
+    turn = 0
+    while any(done[request] < len(tokens) for request, tokens in streams.items()):
+        items = []
+        for request, tokens in streams.items():
+            left = len(tokens) - done[request]
+            if left == 0 or (turn % 3 == 1 and request == "p1"):        # a request may sit a step out
+                continue
+            count = min(left, rng.choice([1, 1, 2, 3, 5, 16, 17, 30]))
+            items.append((request, tokens[done[request]:done[request] + count], [count - 1] if rng.random() < 0.8 else []))
+            done[request] += count
+        if not items:
+            turn += 1
+            continue
+        for replay in (a, b):
+            replay.step(items)
+        if turn % 4 == 2:
+            torch.cuda.synchronize()
+            extra = request_tokens(name, 300 + turn, 9)
+            for replay in (a, b):                         # an eager step in between: every row wanted
+                replay.step([(f"x{turn}", extra, list(range(9)))], end=[f"x{turn}"])
+        turn += 1
+    graphs = recorded.runner._portion_graphs
+    assert len(graphs) >= 2 and all(graph.graph is not None for graph in graphs.values()) and not eager.runner._portion_graphs
+    assert set(a.rows) == set(b.rows) and len(a.rows) > 30
+    keys = sorted(a.rows, key=str)
+    got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
+    bad = first_bad_row(got, want, CUT_TOLERANCE[dtype])
+    assert bad is None, f"replayed step differs from the eager one at {keys[bad]}"
+    # and against the plain implementation
+    for request, tokens in streams.items():
+        places = [key[1] for key in keys if key[0] == request]
+        rows = torch.stack([a.rows[(request, place)] for place in places])
+        assert first_bad_row(rows, plain_logits(setup, tokens)[places], TOLERANCE[dtype]) is None
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
 def test_recorded_decode_steps_replay_like_eager_ones(setups, name, dtype):
     """Decode steps are recorded once per batch-size bucket into a HIP graph and replayed.  Every
     replay is checked against an engine that launches the same steps one kernel at a time, with
@@ -362,6 +412,29 @@ def test_benchmark_layer_sizes_cut_three_ways(tmp_path, dtype):
     engine.finish("p")
     bad = first_bad_row(portions.logits_of("p", range(length)), want, TOLERANCE[dtype])
     assert bad is None, f"portions {sizes}: first wrong position {bad}"
+    # steps that recordings serve (few wanted rows, at most some hundred tokens): two requests cut at
+    # different places, so that a recording is replayed with other portions, with the library's
+    # products at these sizes inside it
+    few = Replayer(engine)
+    cuts = {"q": [100, 78, 12, 110], "r": [90, 90, 1, 119]}
+    starts = {"q": 0, "r": 0}
+    for turn in range(4):
+        items = []
+        for request, sizes in cuts.items():
+            first, size = starts[request], sizes[turn]
+            items.append((request, tokens[first:first + size], [0, size - 1] if size > 1 else [0]))
+            starts[request] += size
+        few.step(items)
+        torch.cuda.synchronize()
+    engine.finish("q")
+    engine.finish("r")
+    graphs = engine.runner._portion_graphs
+    assert (192, 8, 256) in graphs and (16, 8, 256) in graphs and all(graph.graph is not None for graph in graphs.values())
+    for request in cuts:
+        places = sorted(place for name, place in few.rows if name == request)
+        assert len(places) >= 7
+        bad = first_bad_row(few.logits_of(request, places), want[places], TOLERANCE[dtype])
+        assert bad is None, f"recorded portions of {request}: position {places[bad]} is wrong"
 
 
 def plain_sampled_continuation(setup, prompt, generated, temperature, top_p, seed, tolerance):

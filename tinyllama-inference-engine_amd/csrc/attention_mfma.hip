@@ -123,6 +123,7 @@ attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict
   if (tiles != nullptr) {
     const int4 tile = tiles[tile_index];
     seq = tile.x, tok0 = tile.y, ntok = tile.z, col0 = tile.w;
+    if (ntok <= 0) return;                       // a list of fixed size ends in tiles without tokens (the same for the whole workgroup)
   } else {
     const int per_seq = (G + 16 * CT - 1) / (16 * CT);
     seq = tok0 = blockIdx.x / per_seq, ntok = 1, col0 = (blockIdx.x % per_seq) * 16 * CT;

@@ -80,6 +80,9 @@ class Engine:
         self.cache.release(request)
 
     def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
+        """One step of the model: see `ModelRunner.step`.  The logits of a step that is replayed
+        from a recording lie in the recording's memory, which its next replay writes again: copy
+        what has to outlive the next step."""
         return self.runner.step(entries, timings)
 
     # ---- generation -------------------------------------------------------------------------------

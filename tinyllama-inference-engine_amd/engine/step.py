@@ -76,6 +76,9 @@ class StepContext:
     few_rows: bool = False         # at most 16 tokens of bfloat16: the step may use the products that fold norms and adds in
     wants_all_rows: bool = False   # the wanted rows are all the step's tokens, in order
     compute_units: int = 256       # of the device: how many workgroups start at once
+    # a recorded step of prompt portions: its work lists live at fixed addresses, at a fixed size
+    # (the recording's owner makes them: `tiles_for(key, list) -> tensor`); None: a list per step
+    tile_owner: object = None
     _tiles: dict = field(default_factory=dict)
 
     def attention_tiles(self, groups_per_kv: int, num_kv_heads: int, head_dim: int):
@@ -106,7 +109,10 @@ class StepContext:
             def tiles_of(groups):
                 if (groups_per_kv, groups) not in self._tiles:
                     made = attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"])
-                    self._tiles[(groups_per_kv, groups)] = torch.from_numpy(made).to(self.tokens.device)
+                    if self.tile_owner is not None:
+                        self._tiles[(groups_per_kv, groups)] = self.tile_owner.tiles_for((groups_per_kv, groups), made)
+                    else:
+                        self._tiles[(groups_per_kv, groups)] = torch.from_numpy(made).to(self.tokens.device)
                 return self._tiles[(groups_per_kv, groups)]
             tiles = tiles_of(col_tiles * (4 if shared else 1))
             if shared and tiles.shape[0] * num_kv_heads <= 2 * self.compute_units:
@@ -154,6 +160,7 @@ class ModelRunner:
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
         self.device_tokens: torch.Tensor | None = None     # int32, where sampling leaves a step's tokens (set by the engine)
         self._graphs: dict[tuple[int, int], "DecodeGraph"] = {}      # by (most sequences, longest sequence)
+        self._portion_graphs: dict[tuple[int, int, int], "PortionGraph"] = {}   # by (most tokens, most sequences, longest sequence)
 
     # ---- checks and context ------------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]) -> None:
@@ -204,6 +211,21 @@ class ModelRunner:
         return (self.replays_single_tokens(len(entries))
                 and all(len(entry.tokens) == 1 and list(entry.want) == [0] for entry in entries))
 
+    def records(self, entries: Sequence[StepEntry]) -> tuple[int, int] | None:
+        """For a step of prompt portions (beside single tokens, if any) that a recording serves:
+        the recording's (tokens, sequences); else None.  Such steps are bound by the host, which
+        needs some 15 us a launch, up to several hundred tokens; a recording pads the step to its
+        own size, so there are recordings in steps of 64 tokens, up to `PortionGraph.MAX_TOKENS`,
+        for up to 8 or up to 64 sequences, with as many wanted rows as sequences at most."""
+        if not self.use_graphs or any(entry.source is not None for entry in entries):
+            return None
+        total, wanted = sum(len(entry.tokens) for entry in entries), sum(len(entry.want) for entry in entries)
+        if total > PortionGraph.MAX_TOKENS or len(entries) > PortionGraph.MAX_SEQS:
+            return None
+        tokens = 16 if total <= 16 else (32 if total <= 32 else (total + 63) // 64 * 64)
+        seqs = min(tokens, 8 if len(entries) <= 8 else PortionGraph.MAX_SEQS)
+        return (tokens, seqs) if wanted <= seqs else None
+
     # ---- the step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
         """Runs exactly the tokens the entries bring, as one batch, from the cache that earlier
@@ -227,6 +249,12 @@ class ModelRunner:
             if key not in self._graphs:
                 self._graphs[key] = DecodeGraph(self, *key)
             logits = self._graphs[key].run(entries, marks[1] if marks else None)
+        elif (sizes := self.records(entries)) is not None:
+            longest = max(self.cache.length(request) + count for request, count in wanted)
+            key = (*sizes, self._length_bucket(longest))
+            if key not in self._portion_graphs:
+                self._portion_graphs[key] = PortionGraph(self, *key)
+            logits = self._portion_graphs[key].run(entries, marks[1] if marks else None)
         else:
             if any(entry.source is not None for entry in entries):
                 raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
@@ -262,21 +290,25 @@ class DecodeGraph:
             bucket *= 2
         return bucket
 
-    def __init__(self, runner: "ModelRunner", bucket: int, longest: int):
+    def __init__(self, runner: "ModelRunner", bucket: int, longest: int, seqs: int | None = None):
+        # bucket: the recording's tokens; seqs: its sequences (None: as many, one token each).
         # The runner owns its recordings; a recording that owned its runner in turn would make the
         # pair garbage that only the cycle collector frees, at a moment of its choosing: if that
         # moment falls inside another recording's capture, the graph's destructor (which waits for
         # the device) is an operation the capture forbids, and the process ends.
         self._runner = weakref.ref(runner)
         self.bucket = bucket
+        single = seqs is None
+        seqs = bucket if single else seqs
+        self.seqs = seqs
         cache = runner.cache
         self.longest = longest
         self.widths = [max(1, (longest + cache.page_size - 1) // cache.page_size) for _ in cache.groups]
         layout = [("tokens", (bucket,)), ("positions", (bucket,)), ("token_seq", (bucket,)), ("no_slots", (bucket,)),
-                  ("seq_start", (bucket + 1,)), ("seq_first_pos", (bucket,)), ("seq_len", (bucket,)), ("seq_slot", (bucket,)),
-                  ("want_rows", (bucket,)), ("token_source", (bucket,))]
+                  ("seq_start", (seqs + 1,)), ("seq_first_pos", (seqs,)), ("seq_len", (seqs,)), ("seq_slot", (seqs,)),
+                  ("want_rows", (seqs,)), ("token_source", (bucket,))]
         for group, width in enumerate(self.widths):
-            layout += [(f"block_table{group}", (bucket, width)), (f"slot_map{group}", (bucket,))]
+            layout += [(f"block_table{group}", (seqs, width)), (f"slot_map{group}", (bucket,))]
         total = sum(int(np.prod(shape)) for _, shape in layout)
         self.pinned = torch.zeros(total, dtype=torch.int32, pin_memory=True)
         self.device_flat = torch.zeros(total, dtype=torch.int32, device=runner.device)
@@ -287,9 +319,10 @@ class DecodeGraph:
             self.host[name] = flat[cursor:cursor + size].reshape(shape)
             views[name] = self.device_flat[cursor:cursor + size].view(shape)
             cursor += size
-        self.host["token_seq"][:] = np.arange(bucket)
-        self.host["seq_start"][:] = np.arange(bucket + 1)
-        self.host["want_rows"][:] = np.arange(bucket)
+        if single:
+            self.host["token_seq"][:] = np.arange(bucket)
+            self.host["seq_start"][:] = np.arange(bucket + 1)
+            self.host["want_rows"][:] = np.arange(bucket)
         self.host["no_slots"][:] = -1
         self.host["token_source"][:] = -1
         self.token_source = views["token_source"]
@@ -298,11 +331,12 @@ class DecodeGraph:
         groups = [GroupView(views[f"block_table{group}"], views[f"slot_map{group}"], width)
                   for group, width in enumerate(self.widths)]
         self.ctx = StepContext(
-            num_tokens=bucket, num_seqs=bucket, num_wanted=bucket, max_new=1, max_context=longest, tokens=views["tokens"],
-            positions=views["positions"], token_seq=views["token_seq"], no_slots=views["no_slots"],
+            num_tokens=bucket, num_seqs=seqs, num_wanted=seqs, max_new=1 if single else bucket, max_context=longest,
+            tokens=views["tokens"], positions=views["positions"], token_seq=views["token_seq"], no_slots=views["no_slots"],
             seq_start=views["seq_start"], seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"],
             seq_slot=views["seq_slot"], want_rows=views["want_rows"], groups=groups, host=self.host,
-            few_rows=bucket <= 16 and runner.model.dtype == torch.bfloat16, wants_all_rows=True)
+            few_rows=bucket <= 16 and runner.model.dtype == torch.bfloat16, wants_all_rows=single,
+            compute_units=_compute_units(runner.device), tile_owner=None if single else self)
         self.graph = None
         self.logits = None
         self._rows_filled = bucket                           # rows that may hold a step's values
@@ -315,8 +349,9 @@ class DecodeGraph:
             raise invalid_argument("the recording has outlived its runner")
         return runner
 
-    def _fill(self, entries: Sequence[StepEntry]) -> None:
-        """The step's arrays in the pinned buffer.  A row's part of a block table is kept from
+    def _fill(self, entries: Sequence[StepEntry]) -> int:
+        """The step's arrays in the pinned buffer; returns the number of logits rows the step
+        asks for.  A row's part of a block table is kept from
         step to step while the same admission of a request stays in the row: its page list only
         grows, so only the new entries are written.  (Entries of pages that a window has given
         back since keep the old page number: any page number is good there, the kernels mask
@@ -359,6 +394,7 @@ class DecodeGraph:
                 rows.append(page * page_size + (positions[row] & (page_size - 1)))
             slots[:count] = rows
         self._rows_filled = count
+        return count
 
     def run(self, entries: Sequence[StepEntry], transferred=None) -> torch.Tensor:
         """`transferred`: an event to record once the step's arrays are on their way."""
@@ -367,8 +403,9 @@ class DecodeGraph:
             # the pinned buffer is written again only after its last transfer has read it (a caller
             # may run steps without ever waiting for one)
             self.copied.synchronize()
-        self._fill(entries)
+        wanted = self._fill(entries)
         self.device_flat.copy_(self.pinned, non_blocking=True)
+        self._send_lists()
         self.copied.record()
         self.copy_pending = True
         if any(entry.source is not None for entry in entries):
@@ -394,9 +431,86 @@ class DecodeGraph:
                 if collecting:
                     gc.enable()
             self.graph = graph
-            return logits[:len(entries)]
+            return logits[:wanted]
         self.graph.replay()
-        return self.logits[:len(entries)]
+        return self.logits[:wanted]
+
+    def _send_lists(self) -> None:
+        """Work lists that depend on how the step is cut (a decode step has none)."""
+
+
+class PortionGraph(DecodeGraph):
+    """A recorded step of up to `tokens` tokens in up to `seqs` sequences, cut anywhere: portions
+    of prompts beside single tokens, with at most `seqs` wanted rows.  Tokens beyond the step's
+    are padding (token 0 at position 0 of the step's first sequence, written nowhere: slot -1, in
+    no attention tile), sequences beyond the step's have no tokens, wanted rows beyond the step's
+    name row 0; their results are dropped.  The attention kernel's work list has a fixed size
+    too: the tiles of the step, then empty ones."""
+    MAX_TOKENS = 512        # beyond, a step's kernels take longer than the host needs to launch them
+    MAX_SEQS = 64
+
+    def __init__(self, runner: "ModelRunner", tokens: int, seqs: int, longest: int):
+        super().__init__(runner, tokens, longest, seqs=seqs)
+        self._lists: dict = {}            # (group size, column groups) -> (pinned list, the list on the device)
+
+    def tiles_for(self, key, made: np.ndarray) -> torch.Tensor:
+        """The attention work list `key` of this recording, at its fixed place, holding `made`."""
+        if key not in self._lists:
+            if torch.cuda.is_current_stream_capturing():
+                raise invalid_argument("a work list first asked for inside a recording")
+            groups_per_kv, groups = key
+            # a sequence of n tokens has ceil(n * G / (16 * groups)) tiles
+            capacity = (self.bucket * groups_per_kv + 16 * groups - 1) // (16 * groups) + self.seqs
+            self._lists[key] = (torch.zeros((capacity, 4), dtype=torch.int32, pin_memory=True),
+                                torch.zeros((capacity, 4), dtype=torch.int32, device=self.device_flat.device))
+        pinned, device = self._lists[key]
+        if made.shape[0] > pinned.shape[0]:
+            raise invalid_argument(f"{made.shape[0]} attention tiles do not fit the recording's {pinned.shape[0]}")
+        host = pinned.numpy()
+        host[:made.shape[0]] = made
+        host[made.shape[0]:] = 0                                  # no tokens: the kernel leaves at once
+        device.copy_(pinned, non_blocking=True)
+        return device
+
+    def _send_lists(self) -> None:
+        from ..ops import attention_tiles
+        for (groups_per_kv, groups) in self._lists:
+            self.tiles_for((groups_per_kv, groups),
+                           attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"]))
+
+    def _fill(self, entries: Sequence[StepEntry]) -> int:
+        cache, host = self.runner.cache, self.host
+        counts = [len(entry.tokens) for entry in entries]
+        total, seqs = sum(counts), len(entries)
+        first = [cache.length(entry.request) for entry in entries]
+        host["tokens"][:total] = np.concatenate([np.asarray(entry.tokens, dtype=np.int32) for entry in entries])
+        host["tokens"][total:] = 0
+        host["positions"][:total] = np.concatenate([np.arange(start, start + n, dtype=np.int32) for start, n in zip(first, counts)])
+        host["positions"][total:] = 0
+        host["token_seq"][:total] = np.repeat(np.arange(seqs, dtype=np.int32), counts)
+        host["token_seq"][total:] = 0
+        host["seq_start"][0] = 0
+        host["seq_start"][1:seqs + 1] = np.cumsum(counts)
+        host["seq_start"][seqs + 1:] = total
+        host["seq_first_pos"][:seqs] = first
+        host["seq_first_pos"][seqs:] = 0
+        host["seq_len"][:seqs] = [start + n for start, n in zip(first, counts)]
+        host["seq_len"][seqs:] = 1
+        host["seq_slot"][:seqs] = [cache.slot(entry.request) for entry in entries]
+        host["seq_slot"][seqs:] = 0
+        want = [int(host["seq_start"][index]) + int(place) for index, entry in enumerate(entries) for place in entry.want]
+        host["want_rows"][:len(want)] = want
+        host["want_rows"][len(want):] = 0
+        for group in range(len(cache.groups)):
+            table, slots = host[f"block_table{group}"], host[f"slot_map{group}"]
+            table[:] = 0
+            for row, entry in enumerate(entries):
+                pages = cache.page_list(entry.request, group)
+                table[row, :len(pages)] = [page if page != ABSENT else 0 for page in pages]
+            slots[:total] = np.concatenate([np.asarray(cache.rows(entry.request, group, start, n), dtype=np.int32)
+                                            for entry, start, n in zip(entries, first, counts)])
+            slots[total:] = -1
+        return len(want)
 
 
 def _compute_units(device) -> int:
