@@ -552,14 +552,16 @@ def test_a_request_that_stops_at_a_token_beside_one_that_does_not(setups):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype):
+@pytest.mark.parametrize("many", [24, 80])
+def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype, many):
     """The same check for steps of 17 to 24 requests, which take other kernels than small steps do
-    (products that leave partial sums to their consumers): every replay of the recording against
-    the same step launched kernel by kernel, requests ending mid-way."""
+    (products that leave partial sums to their consumers), and of 70 to 80 (the library's products
+    inside the recording): every replay of the recording against the same step launched kernel by
+    kernel, requests ending mid-way."""
     setup = setups("B", dtype)
-    recorded, eager = new_engine(setup, dtype, max_tokens=2048, max_requests=24), \
-        new_engine(setup, dtype, max_tokens=2048, max_requests=24, use_graphs=False)
-    prompts = {f"m{i}": request_tokens("B", 300 + i, 3 + (7 * i) % 23) for i in range(24)}
+    recorded, eager = new_engine(setup, dtype, max_tokens=4096, max_requests=many), \
+        new_engine(setup, dtype, max_tokens=4096, max_requests=many, use_graphs=False)
+    prompts = {f"m{i}": request_tokens("B", 300 + i, 3 + (7 * i) % 23) for i in range(many)}
     follow = {request: request_tokens("B", 400 + i, 12) for i, request in enumerate(prompts)}
     a, b = Replayer(recorded), Replayer(eager)
     for replay in (a, b):
@@ -575,7 +577,8 @@ def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype):
         a.step(items)
         b.step(items)
         torch.cuda.synchronize()
-    assert (32, 256) in recorded.runner._graphs and recorded.runner._graphs[(32, 256)].graph is not None
+    bucket = 32 if many == 24 else 128
+    assert (bucket, 256) in recorded.runner._graphs and recorded.runner._graphs[(bucket, 256)].graph is not None
     keys = sorted(a.rows, key=str)
     assert keys == sorted(b.rows, key=str)
     got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])

@@ -154,9 +154,11 @@ class ModelRunner:
         self.cache = cache
         self.device = model.device
         self.vocab_size = model.spec.vocab_size
-        # Decode steps are bound by launches, not by the kernels: a step of single tokens whose
-        # kernels are all this engine's own is captured once per batch-size bucket and range of
-        # sequence lengths as a HIP graph and replayed.  Parts say whether they may be captured (`graph_safe`).
+        # Steps of up to some hundred tokens are bound by launches, not by the kernels (the host
+        # needs some 15 us a launch, the library's products 20): a step of single tokens is captured
+        # once per batch-size bucket and range of sequence lengths as a HIP graph and replayed, and
+        # so is a step of prompt portions per (tokens, sequences, range of lengths) padded up.
+        # Parts say whether they may be captured (`graph_safe`).
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
         self.device_tokens: torch.Tensor | None = None     # int32, where sampling leaves a step's tokens (set by the engine)
         self._graphs: dict[tuple[int, int], "DecodeGraph"] = {}      # by (most sequences, longest sequence)
@@ -281,7 +283,7 @@ class DecodeGraph:
     How the attention kernel cuts the key range is fixed at capture, for sequences up to
     `longest` positions (the runner keeps a recording per power of two); each part computes its own
     bounds from the positions on the device."""
-    MAX_BATCH = 64          # the largest step whose products all run in this engine's own kernels
+    MAX_BATCH = 256         # beyond, a step's kernels take longer than the host needs to launch them
 
     @staticmethod
     def bucket_of(count: int) -> int:
