@@ -118,6 +118,8 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the configuration has (named in the record)")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
+    parser.add_argument("--prefill", type=int, default=0, metavar="TOKENS",
+                        help="only a prompt step of TOKENS tokens, ten times (for profiles): prints its record alone")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],
                         help="layer sizes of another model of the same architecture (the default is the record's)")
     args = parser.parse_args()
@@ -138,6 +140,13 @@ def main() -> int:
         return 2
     itemsize = 2 if args.dtype == "bfloat16" else 4
     vocab = cfg["vocab_size"]
+    if args.prefill:
+        engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=args.prefill + 2048, page_size=16, max_requests=2)
+        seconds = time_prefill(engine, torch, args.prefill, vocab, repeats=10)
+        print(json.dumps({"metric": f"prefill tok/s at {args.prefill} tokens ({model_name})", "value": args.prefill / seconds,
+                          "unit": "tokens/s", "tokens": args.prefill, "ms": seconds * 1e3,
+                          "frac": prefill_flops(cfg, args.prefill) / seconds / MFMA_PEAK[args.dtype]}))
+        return 0
     most = max(args.batch, 1 if args.no_points else 64)
     engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=most * args.context + 2048,
                     page_size=16, max_requests=most + 1)

@@ -132,6 +132,9 @@ def test_library_product_of_many_rows(shape):
     assert rel_err(got, plain_linear(x.double(), w.double())) < TOL["bfloat16"]
     again = ops.library_mm(x.to(DEV), w.to(DEV))              # the kept plan
     assert torch.equal(got, again)
+    # float32 out (the output head's logits): the sums are not rounded to bfloat16
+    wide = ops.library_mm(x.to(DEV), w.to(DEV), torch.float32)
+    assert wide.dtype == torch.float32 and rel_err(wide, plain_linear(x.double(), w.double())) < 1e-5
 
 
 def test_gemm_is_true_32_bit():

@@ -48,7 +48,7 @@ struct Plan {
 Api api;
 std::mutex guard;
 std::map<int, hipblasLtHandle_t> handles;                              // by device
-std::map<std::tuple<int, int, int, int, size_t>, Plan> plans;         // by (device, M, N, K, workspace)
+std::map<std::tuple<int, int, int, int, int, size_t>, Plan> plans;    // by (device, M, N, K, type of y, workspace)
 #endif
 
 }  // namespace
@@ -82,9 +82,10 @@ extern "C" int tlie_library_gemm_init(const char* path) {
 #endif
 }
 
-// x [M, K], w [N, K], y [M, N]: bfloat16, row-major, dense.  workspace: device memory the library may use.
+// x [M, K], w [N, K]: bfloat16; y [M, N]: bfloat16, or float when y_float != 0 (the sums are float either way);
+// row-major, dense.  workspace: device memory the library may use.
 // Returns 0, or -3 when the library has no algorithm for the shape (or is not there): nothing was launched then.
-extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int M, int N, int K, void* workspace,
+extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_float, int M, int N, int K, void* workspace,
                                  size_t workspace_bytes, void* stream) {
 #ifdef TLIE_HAVE_HIPBLASLT
   if (M <= 0 || N <= 0 || K <= 0) return tlie::kBadArgument;
@@ -98,7 +99,7 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int M, i
     if (api.create(&made) != HIPBLAS_STATUS_SUCCESS) return kUnavailable;
     handle = handles.emplace(device, made).first;
   }
-  const auto key = std::make_tuple(device, M, N, K, workspace_bytes);
+  const auto key = std::make_tuple(device, M, N, K, y_float != 0 ? 1 : 0, workspace_bytes);
   auto found = plans.find(key);
   if (found == plans.end()) {
     // In the library's column-major terms: y^T [N x M] = op_T(W as K x N) . (x as K x M)
@@ -110,7 +111,7 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int M, i
                 api.desc_set(plan.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &plain, sizeof(plain)) == HIPBLAS_STATUS_SUCCESS &&
                 api.layout_create(&plan.w, HIP_R_16BF, K, N, K) == HIPBLAS_STATUS_SUCCESS &&
                 api.layout_create(&plan.x, HIP_R_16BF, K, M, K) == HIPBLAS_STATUS_SUCCESS &&
-                api.layout_create(&plan.y, HIP_R_16BF, N, M, N) == HIPBLAS_STATUS_SUCCESS &&
+                api.layout_create(&plan.y, y_float != 0 ? HIP_R_32F : HIP_R_16BF, N, M, N) == HIPBLAS_STATUS_SUCCESS &&
                 api.preference_create(&preference) == HIPBLAS_STATUS_SUCCESS &&
                 api.preference_set(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
                                    sizeof(workspace_bytes)) == HIPBLAS_STATUS_SUCCESS;
@@ -132,7 +133,7 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int M, i
                                             &plan.algo, workspace, workspace_bytes, (hipStream_t)stream);
   return status == HIPBLAS_STATUS_SUCCESS ? tlie::kOk : tlie::kLaunchFailed;
 #else
-  (void)x, (void)w, (void)y, (void)M, (void)N, (void)K, (void)workspace, (void)workspace_bytes, (void)stream;
+  (void)x, (void)w, (void)y, (void)y_float, (void)M, (void)N, (void)K, (void)workspace, (void)workspace_bytes, (void)stream;
   return kUnavailable;
 #endif
 }

@@ -269,12 +269,14 @@ _library_gemm = {"state": None, "workspace": {}}       # state: None (not tried)
 LIBRARY_WORKSPACE_BYTES = 32 << 20
 
 
-def library_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
-    """y = x . W^T in bfloat16 through the vendor's library (hipBLASLt), for steps of many rows.
-    The library is called directly, with its plan for the shape kept (half the host time of
-    torch.mm, which a step of prompt portions calls four times a layer); where that is not
-    possible (the library's file is not beside torch, or it has no algorithm for the shape)
-    torch.mm makes the same product."""
+def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """y = x . W^T of bfloat16 operands through the vendor's library (hipBLASLt), for steps of many
+    rows; y in bfloat16, or in float32 (the output head's logits).  The library is called
+    directly, with its plan for the shape kept (half the host time of torch.mm, which a step of
+    prompt portions calls four times a layer); where that is not possible (the library's file
+    is not beside torch, or it has no algorithm for the shape) torch.mm makes the same product."""
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise EngineError(ErrorCode.INVALID_DTYPE, f"library_mm gives bfloat16 or float32, not {out_dtype}")
     _device_tensor(x, "x", torch.bfloat16)
     _device_tensor(weight, "weight", torch.bfloat16)
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -290,13 +292,16 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         if index not in state["workspace"]:
             state["workspace"][index] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=x.device)
         workspace = state["workspace"][index]
-        out = torch.empty((x.shape[0], weight.shape[0]), dtype=torch.bfloat16, device=x.device)
-        status = library().tlie_library_gemm(_ptr(x), _ptr(weight), _ptr(out), x.shape[0], weight.shape[0], x.shape[1],
-                                             _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream())
+        out = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=x.device)
+        status = library().tlie_library_gemm(_ptr(x), _ptr(weight), _ptr(out), int(out_dtype == torch.float32), x.shape[0],
+                                             weight.shape[0], x.shape[1], _ptr(workspace), ctypes.c_size_t(workspace.numel()),
+                                             _stream())
         if status == 0:
             return out
         if status != -3:
             _check(status, "library_gemm")
+    if out_dtype == torch.float32:
+        return torch.mm(x.float(), weight.float().t())
     return torch.mm(x, weight.t())
 
 

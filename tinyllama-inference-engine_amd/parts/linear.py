@@ -8,8 +8,9 @@ Which kernel runs is decided here and nowhere else:
                                  product, the SiLU gate or the add into the residual after it
   bfloat16, at most 64 rows      the skinny MFMA kernel (W streamed once, split-K partial sums)
   bfloat16, more rows            the library's product (as the reference uses a library for its
-                                 products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out:
-                                 hipBLASLt called directly (`ops.library_mm`), torch.mm where that fails
+                                 products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out, or
+                                 float32 for the output head: hipBLASLt called directly
+                                 (`ops.library_mm`), torch.mm where that fails
   anything those refuse          the plain kernel
 """
 from __future__ import annotations
@@ -60,10 +61,13 @@ class Linear:
         if ops.gemm_skinny_takes(x, self.weight) and (not whole or out_dtype == torch.float32):
             split_len = (self.in_features + 63) // 64 * 64 if whole else None
             return ops.gemm_skinny(x, self.weight, self.bias, split_len=split_len)
-        if x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16:
+        if x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and out_dtype in (torch.bfloat16, torch.float32):
             ops._device_tensor(x, "x", torch.bfloat16)
             if x.dim() != 2 or x.shape[1] != self.in_features:
                 raise ops.invalid_shape(f"linear: x {list(x.shape)} does not fit weight {list(self.weight.shape)}")
+            if out_dtype == torch.float32:              # (the output head's logits for many rows)
+                out = ops.library_mm(x, self.weight, torch.float32)
+                return Product(out + self.bias.float() if self.bias is not None else out, 1)
             if self.bias is not None:
                 return Product(torch.addmm(self.bias, x, self.weight.t()), 1)
             return Product(ops.library_mm(x, self.weight), 1)
