@@ -392,3 +392,101 @@ def test_toy_parts_register_build_and_step(tmp_path):
     assert_close(replay.logits_of("b", range(23)), want_other, 2e-5, "beside it")
     assert_close(replay.logits_of("c", range(23)), want_other, 2e-5, "in a slot that was used before")
     assert engine.cache.free_slots == 3
+
+
+def register_windowed_toy():
+    """A second architecture of the test's own, out of the framework's parts only: a layer whose
+    attention sees a window of 11 positions (its pages come back while a request runs) and turns
+    half of each head, then a layer whose attention sees everything.  Two page groups; every part
+    may be recorded."""
+    from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run
+    from tlie_amd.registry import register
+
+    @register("architecture", "ToyWindowedForCausalLM")
+    @dataclass(frozen=True)
+    class WindowedConfig:
+        hidden_size: int
+        vocab_size: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["hidden_size"], raw["vocab_size"], raw["eps"])
+
+        def to_dict(self):
+            return {"architectures": ["ToyWindowedForCausalLM"], "hidden_size": self.hidden_size, "vocab_size": self.vocab_size,
+                    "eps": self.eps}
+
+        def to_spec(self):
+            norm = PartSpec("rms_norm", {"size": self.hidden_size, "eps": self.eps})
+
+            def attention(window, rot_dim):
+                position = PartSpec("rotary", {"head_dim": 32, "theta": 300.0, "rot_dim": rot_dim})
+                return PartSpec("attention", {"hidden_size": self.hidden_size, "num_heads": 3, "num_kv_heads": 1, "head_dim": 32,
+                                              "bias": False, "window": window, "position": position})
+            mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 56, "activation": "silu"})
+            layers = (LayerSpec("model.layers.0.", "pre_norm", attention(11, 16), mlp, norm, norm),
+                      LayerSpec("model.layers.1.", "pre_norm", attention(None, 32), mlp, norm, norm))
+            return ModelSpec("ToyWindowedForCausalLM", self.hidden_size, self.vocab_size, 256,
+                             PartSpec("token_embedding", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size}),
+                             layers, (Run(0, 0), Run(1, 1)), norm,
+                             PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "tied": False}))
+    return WindowedConfig
+
+
+def plain_windowed_forward(raw, w, tokens):
+    count, eps = len(tokens), raw["eps"]
+    x = w["model.embed_tokens.weight"][tokens]
+    for layer, (window, rot_dim) in enumerate(((11, 16), (None, 32))):
+        p = f"model.layers.{layer}."
+        normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)
+        x = x + plain_attention_part(normed, w, p + "self_attn.", 3, 1, 32, 300.0, window, False, rot_dim=rot_dim)
+        normed = plain_rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
+        x = x + plain_linear(plain_silu_mul(plain_linear(normed, w[p + "mlp.gate_proj.weight"]),
+                                            plain_linear(normed, w[p + "mlp.up_proj.weight"])), w[p + "mlp.down_proj.weight"])
+    return plain_linear(plain_rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_windowed_architecture_through_recorded_steps(tmp_path, dtype):
+    """Two page groups, one of them windowed, through steps of portions and of single tokens that
+    are replayed from recordings (a block table's entries of pages that the window has given back
+    stay what they were), against the plain implementation; an engine without recordings runs the
+    same steps kernel by kernel."""
+    from tlie_amd import Engine, write_random_model
+    from gpu_helpers import Replayer
+    config = register_windowed_toy()(hidden_size=48, vocab_size=70, eps=1e-5)
+    write_random_model(str(tmp_path), config, seed=9, std=0.15, norm_std=0.1, dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    raw, weights = load_plain(str(tmp_path))
+    tolerance = 2e-5 if dtype == "float32" else 3e-2
+    recorded = Engine(str(tmp_path), dtype=dtype, max_tokens=448, page_size=16, max_requests=3)
+    eager = Engine(str(tmp_path), dtype=dtype, max_tokens=448, page_size=16, max_requests=3, use_graphs=False)
+    assert len(recorded.cache.groups) == 2 and recorded.runner.use_graphs
+    streams = {"u": [(11 * i * i + 5) % 70 for i in range(200)], "v": [(3 * i + 7 * (i % 5)) % 70 for i in range(150)]}
+    want = {request: plain_windowed_forward(raw, weights, tokens) for request, tokens in streams.items()}
+    a, b = Replayer(recorded), Replayer(eager)
+    done = {"u": 0, "v": 0}
+    sizes = [20, 3, 1, 1, 17, 1, 1, 1, 40, 2, 1, 1, 1, 1, 9]
+    turn = 0
+    while any(done[request] < len(streams[request]) for request in streams):
+        items = []
+        for index, request in enumerate(streams):
+            left = len(streams[request]) - done[request]
+            if left == 0:
+                continue
+            count = min(left, sizes[(turn + 4 * index) % len(sizes)])
+            items.append((request, streams[request][done[request]:done[request] + count], [count - 1]))
+            done[request] += count
+        for replay in (a, b):
+            replay.step(items)
+        turn += 1
+    # the windowed group holds two or three pages a request, the other all 13 of the 200 positions
+    held = recorded.cache.held("u").pages
+    assert sum(page >= 0 for page in held[0]) <= 3 and sum(page >= 0 for page in held[1]) == 13
+    assert recorded.runner._graphs and recorded.runner._portion_graphs and not eager.runner._graphs
+    keys = sorted(a.rows, key=str)
+    assert keys == sorted(b.rows, key=str) and len(keys) >= 40
+    for request, tokens in streams.items():
+        places = [place for name, place in keys if name == request]
+        assert_close(a.logits_of(request, places), want[request][places], tolerance, f"{request} recorded")
+        assert_close(b.logits_of(request, places), want[request][places], tolerance, f"{request} eager")
