@@ -80,9 +80,8 @@ class Engine:
         self.cache.release(request)
 
     def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
-        """One step of the model: see `ModelRunner.step`.  The logits of a step that is replayed
-        from a recording lie in the recording's memory, which its next replay writes again: copy
-        what has to outlive the next step."""
+        """One step of the model: see `ModelRunner.step`.  The logits are the caller's own (those
+        of a step replayed from a recording are copied out of the recording's memory)."""
         return self.runner.step(entries, timings)
 
     # ---- generation -------------------------------------------------------------------------------
@@ -145,10 +144,10 @@ class Engine:
                                      [item.count - 1] if item.samples else [], source)
                            for item, source in zip(plan, sources)]
                 if timings is None:
-                    logits = self.step(entries)
+                    logits = self.runner.step(entries, keep=False)
                 else:
                     measured = StepTimings()
-                    logits = self.step(entries, measured)
+                    logits = self.runner.step(entries, measured, keep=False)
                     phase = "decode" if all(item.count == 1 and item.samples and item.request.generated for item in plan) else "prefill"
                     timings[phase + "_compute_ms"] += measured.compute_ms
                     timings[phase + "_transfer_ms"] += measured.transfer_ms

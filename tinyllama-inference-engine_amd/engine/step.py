@@ -229,11 +229,13 @@ class ModelRunner:
         return (tokens, seqs) if wanted <= seqs else None
 
     # ---- the step ----------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, keep: bool = True) -> torch.Tensor:
         """Runs exactly the tokens the entries bring, as one batch, from the cache that earlier
         steps left.  Returns float32 logits [wanted places, vocab] on the device, in the order of
         the entries and of each entry's `want`.  With `timings` the step is timed with events
-        on its stream and waits for them before it returns."""
+        on its stream and waits for them before it returns.  keep=False: the logits may lie in
+        a recording's memory, which the recording's next replay writes again (for a caller that
+        has used them up by then); otherwise they are the caller's own."""
         marks = None
         if timings is not None:
             import time
@@ -251,12 +253,16 @@ class ModelRunner:
             if key not in self._graphs:
                 self._graphs[key] = DecodeGraph(self, *key)
             logits = self._graphs[key].run(entries, marks[1] if marks else None)
+            if keep:
+                logits = logits.clone()
         elif (sizes := self.records(entries)) is not None:
             longest = max(self.cache.length(request) + count for request, count in wanted)
             key = (*sizes, self._length_bucket(longest))
             if key not in self._portion_graphs:
                 self._portion_graphs[key] = PortionGraph(self, *key)
             logits = self._portion_graphs[key].run(entries, marks[1] if marks else None)
+            if keep:
+                logits = logits.clone()
         else:
             if any(entry.source is not None for entry in entries):
                 raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
