@@ -2,6 +2,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 2048] [--dtype bfloat16]
                     [--shape tinyllama|llama2_7b|llama3_8b] [--layers N] [--no-points]
+    python bench.py --workload serving|mixed [--shape ...] [--token-budget 2048]     (records of their own)
+    python bench.py --prefill TOKENS                                                 (a prompt step alone)
 
 A step is one decode step of the whole batch.  The batch's requests are first prefilled so that
 after the warm-up and the K timed steps their length is `context`; then W untimed and exactly K
@@ -108,6 +110,49 @@ def time_prefill(engine, torch, tokens, vocab, repeats=3):
     return best
 
 
+def run_workload(engine, torch, workload, vocab, budget, chunk, slice_steps=8):
+    """A whole workload through the scheduler and the engine's loop, timed in slices of a few
+    steps.  Returns the record's `value` parts and what the scheduler and the cache counted.
+    serving: 64 requests at once, prompts of 128 to 2048 random tokens (or as many as leave the
+    model's positions room for the output), 256 tokens decoded each, continuous batching.  mixed: 8 requests of 8192 positions (prompts of 8176 tokens, 16 decoded), cut into portions of `chunk`, beside 56
+    streams with prompts of 32 to 128 tokens that decode 256 tokens each."""
+    import random
+    from tlie_amd.engine import Request, SamplingParams, Scheduler
+    rng = random.Random(7)
+    generator = torch.Generator().manual_seed(7)
+    if workload == "serving":
+        longest = min(2048, engine.spec.max_positions - 256)           # (a model of 2048 positions: prompts up to 1792)
+        shapes = [(rng.randint(128, longest), 256) for _ in range(64)]
+    else:
+        shapes = [(rng.randint(32, 128), 256) for _ in range(56)] + [(8192 - 16, 16) for _ in range(8)]   # 8192 positions each
+    scheduler = Scheduler(engine.cache, max_tokens_per_step=budget, max_seqs_per_step=len(shapes), chunk_size=chunk,
+                          max_positions=engine.spec.max_positions, eos_token_id=engine.spec.eos_token_id)
+    requests = [Request(id=(workload, index), prompt=torch.randint(0, vocab, (length,), generator=generator).tolist(),
+                        params=SamplingParams(max_tokens=new)) for index, (length, new) in enumerate(shapes)]
+    for request in requests:
+        scheduler.add(request)
+    pages = engine.cache.num_pages
+    slices, peak_pages = [], 0
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    while scheduler.has_work():
+        before = (time.perf_counter(), scheduler.stats["prefill_tokens"])
+        ran = engine.run(scheduler, max_steps=slice_steps)
+        torch.cuda.synchronize()
+        slices.append(((time.perf_counter() - before[0]) / max(ran, 1), scheduler.stats["prefill_tokens"] > before[1]))
+        peak_pages = max(peak_pages, pages - min(engine.cache.free_pages()))
+    elapsed = time.perf_counter() - started
+    assert all(len(request.generated) == new for request, (_, new) in zip(requests, shapes))
+    with_prompts = sorted(seconds for seconds, prompts in slices if prompts)
+    decode_only = sorted(seconds for seconds, prompts in slices if not prompts)
+    middle = lambda values: values[len(values) // 2] * 1e3 if values else None
+    prompt_tokens, new_tokens = sum(length for length, _ in shapes), sum(new for _, new in shapes)
+    return {"seconds": elapsed, "tokens": prompt_tokens + new_tokens, "generated": new_tokens,
+            "steps": scheduler.stats["steps"], "preemptions": scheduler.stats["preemptions"],
+            "peak_pages_frac": peak_pages / pages, "ms_step_with_prompts": middle(with_prompts),
+            "ms_step_decode_only": middle(decode_only)}
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -120,6 +165,11 @@ def main() -> int:
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
     parser.add_argument("--prefill", type=int, default=0, metavar="TOKENS",
                         help="only a prompt step of TOKENS tokens, ten times (for profiles): prints its record alone")
+    parser.add_argument("--workload", default="decode", choices=["decode", "serving", "mixed"],
+                        help="serving: 64 requests with prompts of 128 to 2048 tokens and 256 decoded tokens each, batched "
+                             "continuously; mixed: 8 prompts of 8192 tokens in portions beside 56 short decode streams "
+                             "(needs a shape with 8192 positions); each prints a record of its own")
+    parser.add_argument("--token-budget", type=int, default=2048, help="tokens a step of a workload may hold")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],
                         help="layer sizes of another model of the same architecture (the default is the record's)")
     args = parser.parse_args()
@@ -140,6 +190,22 @@ def main() -> int:
         return 2
     itemsize = 2 if args.dtype == "bfloat16" else 4
     vocab = cfg["vocab_size"]
+    if args.workload != "decode":
+        if args.workload == "mixed" and cfg["max_position_embeddings"] < 8192:
+            print("the mixed workload has prompts of 8192 tokens: take --shape llama3_8b")
+            return 2
+        live = 64 * (2048 + 256) if args.workload == "serving" else 8 * (8192 + 64) + 56 * (128 + 256 + 64)
+        engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=live, page_size=16, max_requests=65)
+        chunk = None if args.workload == "serving" else 512
+        run_workload(engine, torch, args.workload, vocab, args.token_budget, chunk)            # warms up (recordings, plans)
+        got = run_workload(engine, torch, args.workload, vocab, args.token_budget, chunk)
+        print(json.dumps({"metric": f"total tok/s, {args.workload} workload ({model_name})", "value": got["tokens"] / got["seconds"],
+                          "unit": "tokens/s", "generated_per_s": got["generated"] / got["seconds"], "seconds": got["seconds"],
+                          "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "token_budget": args.token_budget,
+                          "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
+                          **{key: got[key] for key in ("steps", "preemptions", "peak_pages_frac", "ms_step_with_prompts",
+                                                       "ms_step_decode_only")}}))
+        return 0
     if args.prefill:
         engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=args.prefill + 2048, page_size=16, max_requests=2)
         seconds = time_prefill(engine, torch, args.prefill, vocab, repeats=10)
