@@ -428,8 +428,8 @@ class DecodeGraph:
             graph = torch.cuda.CUDAGraph()
             # no garbage collection while the capture is open: collecting some dead object that
             # holds device resources (another engine's recording, say) would call into the device
-            # in ways a capture forbids
-            gc.collect()
+            # in ways a capture forbids.  (Switched off, not run beforehand: a collection takes
+            # 20 ms of the 27 that making a recording took with it.)
             collecting = gc.isenabled()
             gc.disable()
             try:
