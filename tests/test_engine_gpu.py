@@ -437,6 +437,46 @@ def test_benchmark_layer_sizes_cut_three_ways(tmp_path, dtype):
         assert bad is None, f"recorded portions of {request}: position {places[bad]} is wrong"
 
 
+# The layer sizes of the two larger shapes that bench.py offers (width 4096, head size 128; one with
+# as many key heads as query heads and a feed-forward of 11008, one with 4 query heads a key head, a
+# feed-forward of 14336 and rope_theta 500000), one layer each and a small vocabulary: other
+# variants of the attention kernels (8 x 16 dims a head, one or four columns a tile in decode
+# steps) and products whose sizes are no multiples of 512.
+LARGER_SHAPES = {
+    "mha_11008": dict(hidden_size=4096, intermediate_size=11008, num_attention_heads=32, num_key_value_heads=32, rope_theta=10000.0),
+    "gqa_14336": dict(hidden_size=4096, intermediate_size=14336, num_attention_heads=32, num_key_value_heads=8, rope_theta=500000.0),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(LARGER_SHAPES))
+def test_larger_layer_sizes_in_bfloat16(tmp_path, shape):
+    raw = dict(BENCH_SHAPE, num_hidden_layers=1, vocab_size=1000, max_position_embeddings=4096, **LARGER_SHAPES[shape])
+    folder = make_model(tmp_path / "model", raw, seed=6, dtype_name="bfloat16", std=0.02, norm_std=0.1)
+    stored, weights = load_plain(folder)
+    length = 150
+    tokens = random_tokens(91, length, 1000)
+    want = plain_forward(stored, weights, tokens)
+    del weights
+    from tlie_amd import Engine
+    engine = Engine(folder, dtype="bfloat16", max_tokens=1024, page_size=16, max_requests=4)
+    whole = Replayer(engine)
+    whole.step([("w", tokens, list(range(length)))], end=["w"])
+    bad = first_bad_row(whole.logits_of("w", range(length)), want, TOLERANCE["bfloat16"])
+    assert bad is None, f"whole prompt: first wrong position {bad}"
+    # a recorded portion, then single tokens beside a second request (recorded decode steps of 2), then portions again
+    cut = Replayer(engine)
+    cut.step([("a", tokens[:97], [96]), ("b", tokens[:97], [0, 96])])
+    for position in range(97, 120):
+        cut.step([("a", [tokens[position]], [0]), ("b", [tokens[position]], [0])])
+    cut.step([("a", tokens[120:], [0, 29]), ("b", tokens[120:137], [16])])
+    cut.step([("b", tokens[137:], [12])], end=["a", "b"])
+    assert engine.runner._graphs and engine.runner._portion_graphs
+    for request in "ab":
+        places = sorted(place for name, place in cut.rows if name == request)
+        bad = first_bad_row(cut.logits_of(request, places), want[places], TOLERANCE["bfloat16"])
+        assert bad is None, f"{shape}: position {places[bad]} of {request} is wrong"
+
+
 def plain_sampled_continuation(setup, prompt, generated, temperature, top_p, seed, tolerance):
     """Checks a sampled continuation against the plain implementation token by token: token i must be
     what the plain distribution at that place gives for the uniform number of (seed, i) when the
