@@ -135,6 +135,16 @@ def test_library_product_of_many_rows(shape):
     # float32 out (the output head's logits): the sums are not rounded to bfloat16
     wide = ops.library_mm(x.to(DEV), w.to(DEV), torch.float32)
     assert wide.dtype == torch.float32 and rel_err(wide, plain_linear(x.double(), w.double())) < 1e-5
+    # recorded: the library's product where it has an algorithm, else the plain kernel (never torch's)
+    xd, wd = x.to(DEV), w.to(DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        recorded = ops.library_mm(xd, wd)
+    for _ in range(3):
+        xd.copy_(torch.randn(m, k).bfloat16())
+        graph.replay()
+        torch.cuda.synchronize()
+        assert rel_err(recorded, plain_linear(xd.double().cpu(), w.double())) < TOL["bfloat16"]
 
 
 def test_gemm_is_true_32_bit():

@@ -274,7 +274,8 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
     rows; y in bfloat16, or in float32 (the output head's logits).  The library is called
     directly, with its plan for the shape kept (half the host time of torch.mm, which a step of
     prompt portions calls four times a layer); where that is not possible (the library's file
-    is not beside torch, or it has no algorithm for the shape) torch.mm makes the same product."""
+    is not beside torch, or it has no algorithm for the shape) torch.mm makes the same product, or,
+    inside a recording, this library's plain kernel."""
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise EngineError(ErrorCode.INVALID_DTYPE, f"library_mm gives bfloat16 or float32, not {out_dtype}")
     _device_tensor(x, "x", torch.bfloat16)
@@ -300,6 +301,10 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
             return out
         if status != -3:
             _check(status, "library_gemm")
+    if torch.cuda.is_current_stream_capturing():
+        # inside a recording no library call that has not been tried there: torch's product may clear a
+        # workspace with a memset node, which replays wrongly; the plain kernel is slow and safe
+        return gemm_generic(x, weight, None, out_dtype).data
     if out_dtype == torch.float32:
         return torch.mm(x.float(), weight.float().t())
     return torch.mm(x, weight.t())

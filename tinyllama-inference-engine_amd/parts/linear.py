@@ -69,6 +69,8 @@ class Linear:
                 out = ops.library_mm(x, self.weight, torch.float32)
                 return Product(out + self.bias.float() if self.bias is not None else out, 1)
             if self.bias is not None:
-                return Product(torch.addmm(self.bias, x, self.weight.t()), 1)
+                # (the bias joins the float32 sums, as in the other kernels; element-wise kernels only, which a
+                # recording can hold: a library product with a bias has not been tried inside one)
+                return Product((ops.library_mm(x, self.weight, torch.float32) + self.bias.float()).to(torch.bfloat16), 1)
             return Product(ops.library_mm(x, self.weight), 1)
         return ops.gemm_generic(x, self.weight, self.bias, out_dtype)
