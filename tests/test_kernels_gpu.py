@@ -82,6 +82,13 @@ def test_silu_mul(dtype):
     got = ops.silu_mul(ops.Product(parts.to(DEV), 2), DT[dtype])
     total = parts.double().sum(0)
     assert rel_err(got, plain_silu_mul(total[:, :177], total[:, 177:])) < TOL[dtype]
+    # a width that takes the kernel with eight results a thread, three summands, both layouts
+    parts = torch.randn(3, 9, 2 * 176) * 2
+    total = parts.double().sum(0)
+    got = ops.silu_mul(ops.Product(parts.to(DEV), 3), DT[dtype])
+    assert rel_err(got, plain_silu_mul(total[:, :176], total[:, 176:])) < TOL[dtype]
+    got = ops.silu_mul(ops.Product(parts.to(DEV), 3), DT[dtype], interleaved=True)
+    assert rel_err(got, plain_silu_mul(total[:, 0::2], total[:, 1::2])) < TOL[dtype]
     extreme = torch.tensor([[80.0, -90.0, 2.0, 2.0]], device=DEV)
     got = ops.silu_mul(ops.Product(extreme, 1), torch.float32).cpu()
     assert got[0, 0] == 160.0 and abs(got[0, 1]) < 1e-30 and torch.isfinite(got).all()

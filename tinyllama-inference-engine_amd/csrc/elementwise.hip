@@ -50,11 +50,12 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const D* __rest
   }
 }
 
-// The same with eight elements a thread (16-byte loads and stores): hidden % 8 == 0, one summand.
+// The same with eight elements a thread (16-byte loads and stores): hidden % 8 == 0; the summands
+// of a split product are added in the order of their index.
 template <typename D, typename W, typename O>
-__global__ void add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* __restrict__ delta,
-                                        const W* __restrict__ weight, float eps, O* __restrict__ out,
-                                        const int* __restrict__ rows, int hidden) {
+__global__ void add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* __restrict__ delta, int nsplit,
+                                        size_t split_stride, const W* __restrict__ weight, float eps,
+                                        O* __restrict__ out, const int* __restrict__ rows, int hidden) {
   extern __shared__ float row_cache[];           // hidden floats, then 16 for the reduction
   float* scratch = row_cache + hidden;
   const int r = blockIdx.x;
@@ -65,8 +66,15 @@ __global__ void add_rmsnorm_wide_kernel(float* __restrict__ residual, const D* _
     float v[8];
     load8(res + i, v);
     if (delta) {
+      const D* part = delta + static_cast<size_t>(src) * hidden + i;
       float d[8];
-      load8(delta + static_cast<size_t>(src) * hidden + i, d);
+      load8(part, d);
+      for (int s = 1; s < nsplit; ++s) {
+        float more[8];
+        load8(part + s * split_stride, more);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) d[j] += more[j];
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] += d[j];
       if (!rows) store8(res + i, v);
@@ -107,10 +115,11 @@ __global__ void silu_mul_kernel(const D* __restrict__ gate_up, int nsplit, size_
   }
 }
 
-// Eight results a thread from sixteen inputs: inter % 8 == 0, one summand.
+// Eight results a thread from sixteen inputs: inter % 8 == 0; the summands of a split product are
+// added in the order of their index.
 template <typename D, typename O>
-__global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, O* __restrict__ out, int rows, int inter,
-                                     int interleaved) {
+__global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, int nsplit, size_t split_stride, O* __restrict__ out,
+                                     int rows, int inter, int interleaved) {
   const int per_row = inter / 8;
   const size_t total = static_cast<size_t>(rows) * per_row;
   for (size_t index = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; index < total;
@@ -119,17 +128,27 @@ __global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, O* __restric
     const int i = static_cast<int>(index % per_row) * 8;
     const D* base = gate_up + t * 2 * inter;
     float a[8], b[8], g[8], u[8];
+    const int first = interleaved ? 2 * i : i, second = interleaved ? 2 * i + 8 : inter + i;
+    load8(base + first, a);
+    load8(base + second, b);
+    for (int s = 1; s < nsplit; ++s) {
+      float more[8];
+      load8(base + s * split_stride + first, more);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a[j] += more[j];
+      load8(base + s * split_stride + second, more);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) b[j] += more[j];
+    }
     if (interleaved) {
-      load8(base + 2 * i, a);
-      load8(base + 2 * i + 8, b);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         g[j] = a[2 * j]; u[j] = a[2 * j + 1];
         g[4 + j] = b[2 * j]; u[4 + j] = b[2 * j + 1];
       }
     } else {
-      load8(base + i, g);
-      load8(base + inter + i, u);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) g[j] = a[j], u[j] = b[j];
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) g[j] = (g[j] / (1.f + expf(-g[j]))) * u[j];
@@ -164,11 +183,11 @@ static int launch_add_rmsnorm(float* residual, const void* delta, int nsplit, si
   if (lds > 160 * 1024) return kBadArgument;
   const bool aligned = ((reinterpret_cast<uintptr_t>(residual) | reinterpret_cast<uintptr_t>(delta) |
                          reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out)) & 31) == 0;
-  if ((hidden & 7) == 0 && nsplit == 1 && aligned) {
+  if ((hidden & 7) == 0 && aligned && (nsplit == 1 || (split_stride * sizeof(D)) % 32 == 0)) {
     const int chunks = hidden / 8;
     const int wide = chunks >= 1024 ? 1024 : (chunks + 63) / 64 * 64;
     hipLaunchKernelGGL((add_rmsnorm_wide_kernel<D, W, O>), dim3(num_rows), dim3(wide), lds, stream, residual,
-                       (const D*)delta, (const W*)weight, eps, (O*)out, rows, hidden);
+                       (const D*)delta, nsplit, split_stride, (const W*)weight, eps, (O*)out, rows, hidden);
     return launch_status();
   }
   const int threads = hidden >= 2048 ? 1024 : (hidden >= 1024 ? 512 : (hidden >= 256 ? 256 : 64));
@@ -207,18 +226,18 @@ extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long
   const int blocks = static_cast<int>(total / threads + 1 < 65536 ? total / threads + 1 : 65536);
   hipStream_t s = (hipStream_t)stream;
   const bool aligned = ((reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(out)) & 31) == 0;
-  if ((inter & 7) == 0 && nsplit == 1 && aligned) {
+  if ((inter & 7) == 0 && aligned && (nsplit == 1 || (in_dtype == kF32 && (split_stride & 7) == 0))) {
     const size_t groups = total / 8;
     const int wide = static_cast<int>(groups / threads + 1 < 65536 ? groups / threads + 1 : 65536);
     if (in_dtype == kF32 && out_dtype == kF32)
       hipLaunchKernelGGL((silu_mul_wide_kernel<float, float>), dim3(wide), dim3(threads), 0, s, (const float*)gate_up,
-                         (float*)out, rows, inter, interleaved);
+                         nsplit, (size_t)split_stride, (float*)out, rows, inter, interleaved);
     else if (in_dtype == kF32 && out_dtype == kBF16)
       hipLaunchKernelGGL((silu_mul_wide_kernel<float, bf16>), dim3(wide), dim3(threads), 0, s, (const float*)gate_up,
-                         (bf16*)out, rows, inter, interleaved);
+                         nsplit, (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
     else if (in_dtype == kBF16 && out_dtype == kBF16)
       hipLaunchKernelGGL((silu_mul_wide_kernel<bf16, bf16>), dim3(wide), dim3(threads), 0, s, (const bf16*)gate_up,
-                         (bf16*)out, rows, inter, interleaved);
+                         nsplit, (size_t)split_stride, (bf16*)out, rows, inter, interleaved);
     else
       return kBadArgument;
     return launch_status();
