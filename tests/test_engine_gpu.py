@@ -208,6 +208,22 @@ def test_greedy_generation_through_the_entry_point(setups, name, dtype):
     assert engine.stats["steps_ahead"] >= 10 and engine.stats["steps_ahead"] <= engine.stats["steps"]
 
 
+def test_greedy_generation_of_a_hundred_requests_at_once(setups):
+    """A hundred requests through the engine's loop in 32-bit: the decode steps are replays of the
+    recording for up to 128 requests, fed with the tokens that sampling left on the device; the
+    token budget admits the prompts over several steps, so requests start and end at different
+    steps.  The tokens of every seventh request are compared with the plain implementation's."""
+    setup = setups("B", "float32")
+    engine = new_engine(setup, "float32", max_tokens=100 * 64, max_requests=100)
+    prompts = [request_tokens("B", 500 + i, 2 + (5 * i) % 19) for i in range(100)]
+    got = engine.generate(prompts, max_tokens=11, max_tokens_per_step=160)
+    assert (128, 256) in engine.runner._graphs
+    for index in range(0, 100, 7):
+        want = plain_generate_greedy(setup["raw"], setup["weights"], prompts[index], 11)
+        assert got[index] == want, f"request {index}"
+    assert engine.cache.free_pages() == [engine.cache.num_pages]
+
+
 @pytest.mark.parametrize("name,dtype", CASES)
 def test_recorded_portion_steps_replay_like_eager_ones(setups, name, dtype):
     """Steps of prompt portions (beside single tokens) of up to some hundred tokens are recorded
