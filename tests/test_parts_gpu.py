@@ -490,3 +490,76 @@ def test_windowed_architecture_through_recorded_steps(tmp_path, dtype):
         places = [place for name, place in keys if name == request]
         assert_close(a.logits_of(request, places), want[request][places], tolerance, f"{request} recorded")
         assert_close(b.logits_of(request, places), want[request][places], tolerance, f"{request} eager")
+
+
+def test_an_embedding_with_learned_positions(tmp_path):
+    """A position encoding of another kind, defined here: a table of learned rows, one per place,
+    added to the token's row by an embedding part of the test's own; the attention then runs with
+    no position encoding of its own.  Whole, in portions and token by token, against the plain
+    functions."""
+    from tlie_amd import Engine, write_random_model
+    from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run, TensorSpec
+    from tlie_amd.parts.base import Part
+    from tlie_amd.registry import register
+    from gpu_helpers import Replayer
+
+    @register("embedding", "toy_token_and_place")
+    class TokenAndPlace(Part):
+        @classmethod
+        def tensor_specs(cls, spec, prefix=""):
+            return [TensorSpec("model.embed_tokens.weight", (spec["vocab_size"], spec["hidden_size"])),
+                    TensorSpec("model.embed_places.weight", (spec["places"], spec["hidden_size"]))]
+
+        def load(self, weights, prefix=""):
+            self.tokens, self.places = weights["model.embed_tokens.weight"], weights["model.embed_places.weight"]
+
+        def forward(self, tokens, ctx):
+            return (self.tokens[tokens.long()].float() + self.places[ctx.positions.long()].float()).contiguous()
+
+    @register("architecture", "ToyPlacesForCausalLM")
+    @dataclass(frozen=True)
+    class PlacesConfig:
+        hidden_size: int
+        vocab_size: int
+        places: int
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["hidden_size"], raw["vocab_size"], raw["places"])
+
+        def to_dict(self):
+            return {"architectures": ["ToyPlacesForCausalLM"], "hidden_size": self.hidden_size, "vocab_size": self.vocab_size,
+                    "places": self.places}
+
+        def to_spec(self):
+            norm = PartSpec("rms_norm", {"size": self.hidden_size, "eps": 1e-5})
+            attention = PartSpec("attention", {"hidden_size": self.hidden_size, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                               "bias": False, "window": None, "position": PartSpec("none")})
+            mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 48, "activation": "silu"})
+            return ModelSpec("ToyPlacesForCausalLM", self.hidden_size, self.vocab_size, self.places,
+                             PartSpec("toy_token_and_place", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+                                                              "places": self.places}),
+                             (LayerSpec("model.layers.0.", "pre_norm", attention, mlp, norm, norm),), (Run(0, 0),), norm,
+                             PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "tied": False}))
+
+    write_random_model(str(tmp_path), PlacesConfig(hidden_size=40, vocab_size=60, places=96), seed=3, std=0.2, norm_std=0.1,
+                       dtype=torch.float32)
+    raw, w = load_plain(str(tmp_path))
+    tokens = [(13 * i * i + 7) % 60 for i in range(70)]
+    x = w["model.embed_tokens.weight"][tokens] + w["model.embed_places.weight"][:70]
+    p = "model.layers.0."
+    x = x + plain_attention_part(plain_rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), w, p + "self_attn.", 4, 2, 16, None, None, False)
+    normed = plain_rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+    x = x + plain_linear(plain_silu_mul(plain_linear(normed, w[p + "mlp.gate_proj.weight"]),
+                                        plain_linear(normed, w[p + "mlp.up_proj.weight"])), w[p + "mlp.down_proj.weight"])
+    want = plain_linear(plain_rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+    engine = Engine(str(tmp_path), dtype="float32", max_tokens=256, page_size=16, max_requests=2)
+    replay = Replayer(engine)
+    replay.step([("whole", tokens, list(range(70)))], end=["whole"])
+    assert_close(replay.logits_of("whole", range(70)), want, 2e-5, "whole")
+    replay.step([("cut", tokens[:33], list(range(33)))])
+    replay.step([("cut", tokens[33:35], [0, 1])])
+    for place in range(35, 70):
+        replay.step([("cut", tokens[place:place + 1], [0])])
+    engine.finish("cut")
+    assert_close(replay.logits_of("cut", range(70)), want, 2e-5, "in portions and token by token")

@@ -67,7 +67,7 @@ class DecoderModel:
             residual, normed = self.embedding.forward_rows(ctx.tokens, first_norm.lazy_params())
             pending = ResidualUpdated(normed)
         else:
-            residual, pending = self.embedding.forward(ctx.tokens), None
+            residual, pending = self.embedding.forward(ctx.tokens, ctx), None
         for index, run in enumerate(runs):
             next_norm = self.blocks[runs[index + 1].layer].mixer_norm if index + 1 < len(runs) else self.final_norm
             pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index], next_norm=next_norm)

@@ -31,7 +31,9 @@ class TokenEmbedding(Part):
     def load(self, weights, prefix=""):
         self.table = weights[self.NAME].contiguous()
 
-    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
+        """The float32 residual [T, H] of the step's tokens.  `ctx` is the step's context: an
+        embedding that depends on more than the token (positions learned per place, say) reads it."""
         return ops.embed_gather(tokens, self.table)
 
     def forward_rows(self, tokens: torch.Tensor, next_norm: tuple):
