@@ -138,3 +138,22 @@ def test_sharded_folder(tmp_path):
     (tmp_path / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
     loaded = WeightStore(str(tmp_path)).load(specs, torch.float32, "cpu")
     assert all(torch.equal(loaded[n], tensors[n].float()) for n in names)
+
+
+def test_checksum_of_the_weight_file(tmp_path):
+    """The reference checks its weights against a pinned digest (`checksum_mismatch`,
+    tests/unit_tests.cpp:150-160); here the digest is the caller's to name."""
+    import hashlib
+    from tlie_amd import EngineError, LlamaConfig, write_random_model
+    from tlie_amd.weights import WeightStore
+    raw = dict(model_type="llama", hidden_size=32, intermediate_size=48, num_hidden_layers=1, num_attention_heads=2,
+               num_key_value_heads=1, max_position_embeddings=32, vocab_size=40, rms_norm_eps=1e-5)
+    write_random_model(str(tmp_path), LlamaConfig.from_dict(raw), seed=1)
+    with open(tmp_path / "model.safetensors", "rb") as handle:
+        digest = hashlib.sha256(handle.read()).hexdigest()
+    store = WeightStore(str(tmp_path))
+    assert store.sha256() == digest
+    store.expect_sha256(digest.upper() + "\n")
+    with pytest.raises(EngineError) as caught:
+        store.expect_sha256("0" * 64)
+    assert caught.value.code.value == "checksum_mismatch"

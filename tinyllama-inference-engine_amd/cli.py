@@ -27,7 +27,8 @@ USAGE = ("usage: tinyllama_amd generate MODEL_DIR PROMPT MAX_TOKENS [GOLDEN_JSON
          "       tinyllama_amd logits MODEL_DIR PROMPT\n"
          "       tinyllama_amd benchmark MODEL_DIR CONTEXT OUTPUT_TOKENS WARMUP SAMPLES\n"
          "       tinyllama_amd random MODEL_DIR CONFIG_JSON SEED\n"
-         "options: [--dtype bfloat16|float32] [--temperature T] [--top-p P] [--seed S] [--max-cache-tokens N]\n")
+         "options: [--dtype bfloat16|float32] [--temperature T] [--top-p P] [--seed S] [--max-cache-tokens N]\n"
+         "         [--expect-sha256 HEX]\n")
 
 
 def parse_integer(text: str, name: str, minimum: int) -> int:
@@ -60,7 +61,7 @@ def prompt_ids(model_dir: str, prompt: str) -> tuple[list[int], object]:
 def _engine(args, positions: int):
     from .engine import Engine
     return Engine(args.model_dir, dtype=args.dtype, max_tokens=args.max_cache_tokens or max(64, positions),
-                  max_requests=4)
+                  max_requests=4, expect_sha256=args.expect_sha256)
 
 
 def command_generate(args) -> int:
@@ -168,6 +169,7 @@ def main(argv=None) -> int:
     parser.add_argument("--top-p", type=float, default=1.0)
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--max-cache-tokens", type=int, default=0)
+    parser.add_argument("--expect-sha256", default=None)
     try:
         options, positional = parser.parse_known_args(argv)
     except SystemExit:

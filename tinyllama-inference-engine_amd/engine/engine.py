@@ -39,12 +39,13 @@ def parse_dtype(name) -> torch.dtype:
 class Engine:
     def __init__(self, model_dir: str | None, dtype="bfloat16", max_tokens: int = 4096, page_size: int = 16,
                  max_requests: int = 64, device: str = "cuda:0", config: dict | None = None,
-                 random_seed: int | None = None, use_graphs: bool = True):
+                 random_seed: int | None = None, use_graphs: bool = True, expect_sha256: str | None = None):
         """max_tokens: how many positions the cache pools hold in all (rounded up to whole
         pages); max_requests: how many requests can be live at once.
 
         Without a folder, `config` (the contents of a config.json) and `random_seed` give a model
-        of random weights drawn on the device, with no file in between (for measurements)."""
+        of random weights drawn on the device, with no file in between (for measurements).
+        expect_sha256: the digest the folder's weight file must have (`checksum_mismatch` otherwise)."""
         if not torch.cuda.is_available():
             raise EngineError(ErrorCode.HIP, "no GPU is visible: the engine has no CPU path")
         self.dtype = parse_dtype(dtype)
@@ -53,7 +54,10 @@ class Engine:
         if model_dir is not None:
             self.config = config_from_dict(read_config_json(model_dir))
             self.spec = self.config.to_spec()
-            weights = WeightStore(model_dir).load(expected_tensors(self.spec), self.dtype, self.device)
+            store = WeightStore(model_dir)
+            if expect_sha256 is not None:
+                store.expect_sha256(expect_sha256)
+            weights = store.load(expected_tensors(self.spec), self.dtype, self.device)
         else:
             if config is None or random_seed is None:
                 raise invalid_argument("without a model folder the engine needs a config and a random seed")

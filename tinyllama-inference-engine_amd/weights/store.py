@@ -54,6 +54,25 @@ class WeightStore:
                     raise EngineError(ErrorCode.INVALID_FORMAT, f"tensor '{tensor_name}' is stored in two files")
                 self._where[tensor_name] = file
 
+    def sha256(self) -> str:
+        """The SHA-256 of the weight files' bytes, in the order of their names (one file: that
+        file's digest, as `sha256sum model.safetensors` prints it)."""
+        import hashlib
+        digest = hashlib.sha256()
+        for file in self._files:
+            with open(file.path, "rb") as handle:
+                for block in iter(lambda: handle.read(1 << 24), b""):
+                    digest.update(block)
+        return digest.hexdigest()
+
+    def expect_sha256(self, expected: str) -> None:
+        """reference: the weights' digest is a pinned trust root there, checked at load
+        (include/tlie/pinned_model.hpp:7-14, src/weight_store.cpp:162-165: `checksum_mismatch`);
+        here the caller may name one."""
+        found = self.sha256()
+        if found != expected.strip().lower():
+            raise EngineError(ErrorCode.CHECKSUM_MISMATCH, f"the weights' SHA-256 is {found}, expected {expected.strip().lower()}")
+
     def names(self) -> list[str]:
         return sorted(self._where)
 
