@@ -106,3 +106,16 @@ def test_error_json_shape():
     names = {code.value for code in ErrorCode}
     assert {"io_error", "invalid_format", "checksum_mismatch", "invalid_config", "invalid_shape", "invalid_dtype",
             "out_of_memory", "out_of_bounds", "tokenizer_error", "numerical_error", "invalid_argument"} <= names
+
+
+def test_the_device_allocators_refusal_is_out_of_memory():
+    """reference: a failed device allocation is `out_of_memory` (src/cuda/weight_store.cpp:273-274)."""
+    import torch
+    from tlie_amd.errors import EngineError, device_memory_errors
+    with pytest.raises(EngineError) as caught:
+        with device_memory_errors("the cache pools"):
+            raise torch.cuda.OutOfMemoryError("tried to allocate 1 TiB")
+    assert caught.value.code.value == "out_of_memory" and "cache pools" in caught.value.message
+    with pytest.raises(KeyError):                      # anything else passes through
+        with device_memory_errors("the weights"):
+            raise KeyError("x")

@@ -15,7 +15,7 @@ import torch
 from .. import models as _models  # noqa: F401  (registers architectures and parts)
 from ..cache.manager import CacheManager
 from ..config.llama import read_config_json
-from ..errors import EngineError, ErrorCode, invalid_argument
+from ..errors import EngineError, ErrorCode, device_memory_errors, invalid_argument
 from ..models.builder import build_model, expected_tensors
 from ..registry import config_from_dict
 from ..weights.store import WeightStore
@@ -57,20 +57,24 @@ class Engine:
             store = WeightStore(model_dir)
             if expect_sha256 is not None:
                 store.expect_sha256(expect_sha256)
-            weights = store.load(expected_tensors(self.spec), self.dtype, self.device)
+            with device_memory_errors("the weights"):
+                weights = store.load(expected_tensors(self.spec), self.dtype, self.device)
         else:
             if config is None or random_seed is None:
                 raise invalid_argument("without a model folder the engine needs a config and a random seed")
             from ..weights.random_init import random_tensors
             self.config = config_from_dict(config)
             self.spec = self.config.to_spec()
-            weights = random_tensors(expected_tensors(self.spec), random_seed, dtype=self.dtype, device=self.device)
-        self.model = build_model(self.spec, weights, self.dtype, self.device)
+            with device_memory_errors("the weights"):
+                weights = random_tensors(expected_tensors(self.spec), random_seed, dtype=self.dtype, device=self.device)
+        with device_memory_errors("the weights"):
+            self.model = build_model(self.spec, weights, self.dtype, self.device)
         if max_tokens <= 0:
             raise invalid_argument("max_tokens must be positive")
         num_pages = (max_tokens + page_size - 1) // page_size
-        self.cache = CacheManager(self.model.run_needs(), page_size, num_pages, max_requests, self.dtype, self.device,
-                                  max_positions=self.spec.max_positions)
+        with device_memory_errors(f"cache pools of {num_pages} pages"):
+            self.cache = CacheManager(self.model.run_needs(), page_size, num_pages, max_requests, self.dtype, self.device,
+                                      max_positions=self.spec.max_positions)
         self.runner = ModelRunner(self.model, self.cache, use_graphs=use_graphs)
         self.sampler = Sampler(self.device, capacity=max(max_requests, 1))
         self.runner.device_tokens = self.sampler.device_tokens

@@ -56,3 +56,21 @@ def out_of_bounds(message: str) -> EngineError:
 
 def out_of_memory(message: str) -> EngineError:
     return EngineError(ErrorCode.OUT_OF_MEMORY, message)
+
+
+class device_memory_errors:
+    """`with device_memory_errors("the cache pools"):` turns the device allocator's refusal into
+    `out_of_memory`, as the reference maps a failed device allocation of its weights and of its
+    cache (src/cuda/weight_store.cpp:273-274, src/cuda/model.cu:262-270)."""
+
+    def __init__(self, what: str):
+        self.what = what
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, kind, error, traceback):
+        import torch
+        if kind is not None and issubclass(kind, torch.cuda.OutOfMemoryError):
+            raise EngineError(ErrorCode.OUT_OF_MEMORY, f"the device has no memory for {self.what}: {error}") from None
+        return False
