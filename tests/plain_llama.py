@@ -142,8 +142,15 @@ def plain_top_p_distribution(logits: torch.Tensor, temperature: float, top_p: fl
     return out / out.sum()
 
 
-def plain_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, cfg: dict) -> torch.Tensor:
-    """One pre-norm block: x + attn(norm(x)), then x + mlp(norm(x)).  src/model.cpp:132-203."""
+def plain_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, cfg: dict, trace: dict | None = None,
+                trace_prefix: str = "") -> torch.Tensor:
+    """One pre-norm block: x + attn(norm(x)), then x + mlp(norm(x)).  src/model.cpp:132-203.
+    `trace` receives the five tensors the reference's ModelTrace keeps per layer
+    (src/model.cpp:136-138,176-177,184-185,200-201,204-205)."""
+    def keep(name, tensor):
+        if trace is not None:
+            trace[trace_prefix + name] = tensor
+
     heads = cfg["num_attention_heads"]
     kv_heads = cfg.get("num_key_value_heads", heads)
     head_dim = cfg.get("head_dim", cfg["hidden_size"] // heads)
@@ -154,35 +161,49 @@ def plain_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, 
         return w.get(prefix + name)
 
     normed = plain_rms_norm(x, w[prefix + "input_layernorm.weight"], eps)
+    keep("input_norm", normed)
     q = plain_linear(normed, w[prefix + "self_attn.q_proj.weight"], bias("self_attn.q_proj.bias"))
     k = plain_linear(normed, w[prefix + "self_attn.k_proj.weight"], bias("self_attn.k_proj.bias"))
     v = plain_linear(normed, w[prefix + "self_attn.v_proj.weight"], bias("self_attn.v_proj.bias"))
     q = plain_rope(q.view(tokens, heads, head_dim), positions, theta)
     k = plain_rope(k.view(tokens, kv_heads, head_dim), positions, theta)
     attended = plain_attention(q, k, v.view(tokens, kv_heads, head_dim))
-    x = x + plain_linear(attended.reshape(tokens, heads * head_dim),
-                         w[prefix + "self_attn.o_proj.weight"], bias("self_attn.o_proj.bias"))
+    projected = plain_linear(attended.reshape(tokens, heads * head_dim),
+                             w[prefix + "self_attn.o_proj.weight"], bias("self_attn.o_proj.bias"))
+    keep("attention_output", projected)
+    x = x + projected
     normed = plain_rms_norm(x, w[prefix + "post_attention_layernorm.weight"], eps)
+    keep("post_attention_norm", normed)
     gate = plain_linear(normed, w[prefix + "mlp.gate_proj.weight"])
     up = plain_linear(normed, w[prefix + "mlp.up_proj.weight"])
-    return x + plain_linear(plain_silu_mul(gate, up), w[prefix + "mlp.down_proj.weight"])
+    projected = plain_linear(plain_silu_mul(gate, up), w[prefix + "mlp.down_proj.weight"])
+    keep("mlp_output", projected)
+    keep("output", x + projected)
+    return x + projected
 
 
-def plain_forward(cfg: dict, w: dict, tokens: list[int], first_position: int = 0) -> torch.Tensor:
+def plain_forward(cfg: dict, w: dict, tokens: list[int], first_position: int = 0, trace: dict | None = None) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.  src/model.cpp:80-234.
 
     Embedding row copy (:94-97), the blocks in order (:112-207), final norm (:217) and the
     output projection (:224-225); with tied embeddings the output projection is the
     embedding table.  `first_position` shifts every position; it is for the tests' invariants.
+    `trace` receives the named tensors of the reference's ModelTrace ("embedding", "layerN.*",
+    "final_norm", "logits": src/model.cpp:98-99,221-222,229-230).
     """
     ids = torch.tensor(tokens, dtype=torch.long)
     positions = torch.arange(len(tokens)) + first_position
     x = w["model.embed_tokens.weight"].double()[ids]
+    if trace is not None:
+        trace["embedding"] = x
     for layer in range(cfg["num_hidden_layers"]):
-        x = plain_block(x, positions, w, f"model.layers.{layer}.", cfg)
+        x = plain_block(x, positions, w, f"model.layers.{layer}.", cfg, trace, f"layer{layer}.")
     normed = plain_rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
-    return plain_linear(normed, head)
+    logits = plain_linear(normed, head)
+    if trace is not None:
+        trace["final_norm"], trace["logits"] = normed, logits
+    return logits
 
 
 def plain_generate_greedy(cfg: dict, w: dict, prompt: list[int], max_tokens: int) -> list[int]:

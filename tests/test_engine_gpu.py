@@ -64,6 +64,41 @@ def test_whole_and_alone(setups, name, dtype):
 
 
 @pytest.mark.parametrize("name,dtype", CASES)
+def test_named_intermediate_tensors_layer_by_layer(setups, name, dtype):
+    """The reference compares its model with a golden layer by layer through a trace of named
+    tensors (ModelTrace: src/model.cpp:98-231, tests/m1_integration_tests.cpp:92-128).  A step that
+    is given a dict leaves the same names there; each is compared with the plain implementation's,
+    so that a fault shows in the first tensor it touches.  A prompt in two portions: the second
+    portion's rows are the sequence's later positions."""
+    setup = setups(name, dtype)
+    engine = new_engine(setup, dtype)
+    tokens = request_tokens(name, 3, 45)
+    plain = {}
+    plain_forward(setup["raw"], setup["weights"], tokens, trace=plain)
+    layers = CONFIGS[name]["num_hidden_layers"]
+    assert len(plain) == 5 * layers + 3
+    from tlie_amd import StepEntry
+    engine.admit("t")
+    first, second = {}, {}
+    engine.step([StepEntry("t", tokens[:30], list(range(30)))], trace=first)
+    engine.step([StepEntry("t", tokens[30:], list(range(15)))], trace=second)
+    engine.finish("t")
+    assert sorted(first) == sorted(plain) == sorted(second)
+    order = ["embedding"] + [f"layer{layer}.{part}" for layer in range(layers)
+                             for part in ("input_norm", "attention_output", "post_attention_norm", "mlp_output", "output")] \
+        + ["final_norm", "logits"]
+    for key in order:
+        got = torch.cat([first[key], second[key]]).cpu()
+        assert got.dtype == torch.float32 and got.shape == plain[key].shape, key
+        assert_close(got, plain[key], TOLERANCE[dtype], key)
+    # a step without a dict is not slowed or changed by all this: the same logits
+    engine.admit("u")
+    again = engine.step([StepEntry("u", tokens, list(range(45)))]).cpu()
+    engine.finish("u")
+    assert_close(again, torch.cat([first["logits"], second["logits"]]).cpu().double(), CUT_TOLERANCE[dtype], "without a trace")
+
+
+@pytest.mark.parametrize("name,dtype", CASES)
 def test_most_in_one_step_then_the_last_32_one_by_one(setups, name, dtype):
     setup = setups(name, dtype)
     engine = new_engine(setup, dtype)

@@ -214,3 +214,22 @@ def test_model_bias_is_applied_before_rotation():
     cfg, w = _tiny(seed=5, bias=True)
     cfg = dict(cfg, num_hidden_layers=1)
     assert not torch.allclose(plain_forward(cfg, w, [1, 2, 3])[2], plain_forward(cfg, {**w, "model.layers.0.self_attn.k_proj.bias": torch.zeros(8)}, [1, 2, 3])[2], atol=1e-6)
+
+
+def test_model_trace_names_and_the_residual_sums():
+    """The named tensors of the reference's ModelTrace (src/model.cpp:98-231): 5 a layer + 3 (113
+    for its 22 layers, scripts/export_golden.py:73-107), and what ties them together: a layer's
+    output is its input plus its two projected outputs."""
+    cfg, w = _tiny(seed=2)
+    tokens = [4, 8, 15, 16, 23, 42]
+    trace = {}
+    logits = plain_forward(cfg, w, tokens, trace=trace)
+    assert len(trace) == 5 * 2 + 3 and torch.equal(trace["logits"], logits)
+    assert torch.equal(trace["embedding"], w["model.embed_tokens.weight"].double()[tokens])
+    before = trace["embedding"]
+    for layer in range(2):
+        p = f"layer{layer}."
+        assert torch.allclose(trace[p + "output"], before + trace[p + "attention_output"] + trace[p + "mlp_output"], atol=1e-12)
+        assert torch.allclose(trace[p + "input_norm"], plain_rms_norm(before, w[f"model.layers.{layer}.input_layernorm.weight"], 1e-5))
+        before = trace[p + "output"]
+    assert torch.allclose(trace["final_norm"], plain_rms_norm(before, w["model.norm.weight"], 1e-5))

@@ -87,10 +87,11 @@ class Engine:
     def finish(self, request: Hashable) -> None:
         self.cache.release(request)
 
-    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, trace: dict | None = None) -> torch.Tensor:
         """One step of the model: see `ModelRunner.step`.  The logits are the caller's own (those
-        of a step replayed from a recording are copied out of the recording's memory)."""
-        return self.runner.step(entries, timings)
+        of a step replayed from a recording are copied out of the recording's memory).  `trace`: a
+        dict that receives the step's intermediate tensors by the names of the reference's ModelTrace."""
+        return self.runner.step(entries, timings, trace=trace)
 
     # ---- generation -------------------------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,

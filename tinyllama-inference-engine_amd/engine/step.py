@@ -79,6 +79,10 @@ class StepContext:
     # a recorded step of prompt portions: its work lists live at fixed addresses, at a fixed size
     # (the recording's owner makes them: `tiles_for(key, list) -> tensor`); None: a list per step
     tile_owner: object = None
+    # a dict that receives named copies of the step's intermediate tensors (such a step is never
+    # replayed from a recording and takes no fused route), and the name's prefix for the layer that runs
+    trace: dict | None = None
+    trace_prefix: str = ""
     _tiles: dict = field(default_factory=dict)
 
     def attention_tiles(self, groups_per_kv: int, num_kv_heads: int, head_dim: int):
@@ -229,13 +233,16 @@ class ModelRunner:
         return (tokens, seqs) if wanted <= seqs else None
 
     # ---- the step ----------------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, keep: bool = True) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, keep: bool = True,
+             trace: dict | None = None) -> torch.Tensor:
         """Runs exactly the tokens the entries bring, as one batch, from the cache that earlier
         steps left.  Returns float32 logits [wanted places, vocab] on the device, in the order of
         the entries and of each entry's `want`.  With `timings` the step is timed with events
         on its stream and waits for them before it returns.  keep=False: the logits may lie in
         a recording's memory, which the recording's next replay writes again (for a caller that
-        has used them up by then); otherwise they are the caller's own."""
+        has used them up by then); otherwise they are the caller's own.  trace: a dict that
+        receives the step's intermediate tensors by name (see `DecoderModel.forward`); the step
+        is then launched kernel by kernel."""
         marks = None
         if timings is not None:
             import time
@@ -247,7 +254,7 @@ class ModelRunner:
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
         if marks:
             marks[0].record()
-        if self.replays(entries):
+        if trace is None and self.replays(entries):
             longest = max(self.cache.length(request) + count for request, count in wanted)
             key = (DecodeGraph.bucket_of(len(entries)), self._length_bucket(longest))
             if key not in self._graphs:
@@ -255,7 +262,7 @@ class ModelRunner:
             logits = self._graphs[key].run(entries, marks[1] if marks else None)
             if keep:
                 logits = logits.clone()
-        elif (sizes := self.records(entries)) is not None:
+        elif trace is None and (sizes := self.records(entries)) is not None:
             longest = max(self.cache.length(request) + count for request, count in wanted)
             key = (*sizes, self._length_bucket(longest))
             if key not in self._portion_graphs:
@@ -267,6 +274,7 @@ class ModelRunner:
             if any(entry.source is not None for entry in entries):
                 raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
             ctx = self.build_context(entries)
+            ctx.trace = trace
             if marks:
                 marks[1].record()
             logits = self.model.forward(ctx, self.cache.bindings)

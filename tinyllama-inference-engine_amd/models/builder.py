@@ -60,24 +60,38 @@ class DecoderModel:
         return needs
 
     def forward(self, ctx, bindings) -> torch.Tensor:
-        """Runs the step's tokens; returns float32 logits [wanted rows, vocab]."""
+        """Runs the step's tokens; returns float32 logits [wanted rows, vocab].  With `ctx.trace` (a
+        dict) the named tensors of the reference's ModelTrace are left there as float32 copies:
+        "embedding", per run i "layer{i}.input_norm", ".attention_output", ".post_attention_norm",
+        ".mlp_output", ".output", then "final_norm" and "logits" at the wanted rows
+        (src/model.cpp:98-231)."""
         runs = self.spec.runs
+        trace = getattr(ctx, "trace", None)
         first_norm = self.blocks[runs[0].layer].mixer_norm
-        if ctx.few_rows and hasattr(self.embedding, "forward_rows") and first_norm.lazy_params() is not None:
+        if (ctx.few_rows and trace is None and hasattr(self.embedding, "forward_rows")
+                and first_norm.lazy_params() is not None):
             residual, normed = self.embedding.forward_rows(ctx.tokens, first_norm.lazy_params())
             pending = ResidualUpdated(normed)
         else:
             residual, pending = self.embedding.forward(ctx.tokens, ctx), None
+        if trace is not None:
+            trace["embedding"] = residual.float().clone()
         for index, run in enumerate(runs):
             next_norm = self.blocks[runs[index + 1].layer].mixer_norm if index + 1 < len(runs) else self.final_norm
+            if trace is not None:
+                ctx.trace_prefix = f"layer{index}."
             pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index], next_norm=next_norm)
         if ctx.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if ctx.wants_all_rows:
-            normed = self.final_norm.add_forward(residual, pending, lazy=ctx.few_rows and self.head.takes_normed_rows(residual.shape[0]))
+            lazy = ctx.few_rows and trace is None and self.head.takes_normed_rows(residual.shape[0])
+            normed = self.final_norm.add_forward(residual, pending, lazy=lazy)
         else:
             normed = self.final_norm.add_forward(residual, pending, rows=ctx.want_rows)
-        return self.head.forward(normed)
+        logits = self.head.forward(normed)
+        if trace is not None:
+            trace["final_norm"], trace["logits"] = normed.float().clone(), logits.clone()
+        return logits
 
 
 def build_model(spec: ModelSpec, weights: dict[str, torch.Tensor], dtype: torch.dtype, device) -> DecoderModel:

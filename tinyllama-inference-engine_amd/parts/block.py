@@ -8,7 +8,10 @@ the model's final norm) adds it in the same kernel.
 """
 from __future__ import annotations
 
+import torch
+
 from ..config.spec import LayerSpec
+from ..ops import ResidualUpdated, as_product
 from ..registry import lookup, register
 from .base import ResidualTarget
 
@@ -49,7 +52,12 @@ class PreNormBlock:
         """`pending`: what the residual still lacks (a product, a `ResidualUpdated`, or None).
         `next_norm`: the norm that reads the residual after this block, if the caller knows it.
         In a step of few rows the parts that offer it fold the norms into their products and add
-        their results into the residual themselves; otherwise the norm kernels do both."""
+        their results into the residual themselves; otherwise the norm kernels do both.
+        A step that keeps a trace (`ctx.trace`, a dict) takes the second way and leaves there, under
+        `ctx.trace_prefix`, the five tensors the reference's ModelTrace keeps per layer
+        (src/model.cpp:136-138,176-177,184-185,200-201,204-205), as float32 copies."""
+        if getattr(ctx, "trace", None) is not None:
+            return self._forward_traced(residual, pending, ctx, binding)
         rows = residual.shape[0]
         few = ctx.few_rows
         normed = self.mixer_norm.add_forward(residual, pending, lazy=few and self.mixer.takes_normed_rows(rows))
@@ -62,3 +70,20 @@ class PreNormBlock:
             return self.feed_forward.forward(normed, ctx, into=ResidualTarget(
                 residual, next_norm.lazy_params() if next_norm is not None else None))
         return self.feed_forward.forward(normed, ctx)
+
+    def _forward_traced(self, residual, pending, ctx, binding):
+        def keep(name, tensor):
+            ctx.trace[ctx.trace_prefix + name] = tensor.float().clone()
+
+        def dense(result):
+            return as_product(result).dense(torch.float32)
+        normed = self.mixer_norm.add_forward(residual, pending)
+        keep("input_norm", normed)
+        mixed = self.mixer.forward(normed, ctx, binding)
+        keep("attention_output", dense(mixed))
+        normed = self.feed_forward_norm.add_forward(residual, mixed)
+        keep("post_attention_norm", normed)
+        out = self.feed_forward.forward(normed, ctx)
+        keep("mlp_output", dense(out))
+        keep("output", residual + dense(out))
+        return out
