@@ -415,6 +415,19 @@ def test_replay_program_and_command_line(setups, tmp_path):
     assert run.returncode != 0 and error_code(run.stderr) == "tokenizer_error"
     run = subprocess.run(cli + ["generate", setup["folder"], prompt, "200"], capture_output=True, text=True, timeout=300)
     assert run.returncode != 0 and error_code(run.stderr) == "out_of_bounds"         # app/reference_cli.cpp:72-75
+    # benchmark MODEL_DIR CONTEXT OUTPUT_TOKENS WARMUP SAMPLES, with the reference's keys (app/cuda_reference.cu:435-469)
+    run = subprocess.run(cli + ["benchmark", setup["folder"], "20", "5", "1", "2", "--dtype", "float32"], capture_output=True, text=True,
+                         timeout=300)
+    assert run.returncode == 0, run.stderr
+    result = json.loads(run.stdout)
+    assert result["schema_version"] == 1 and result["context"] == 20 and result["output_tokens"] == 5 and result["sample_count"] == 2
+    assert len(result["samples"]) == 2 and all(row["ttft_ms"] > 0 and row["tpot_ms"] > 0 for row in result["samples"])
+    assert len(result["generated_tokens"]) == 5 and result["sampling"] == "greedy" and result["batch"] == 1
+    assert 0 < result["kv_cache_bytes"] < result["engine_peak_device_bytes"] <= result["vram_bytes"] and result["model_device_bytes"] > 0
+    assert result["device_segments_after_workload"] >= result["device_segments_before_workload"] > 0
+    # the digest of the weight file, when the caller names one
+    run = subprocess.run(cli + ["logits", setup["folder"], prompt, "--expect-sha256", "ab" * 32], capture_output=True, text=True, timeout=300)
+    assert run.returncode != 0 and error_code(run.stderr) == "checksum_mismatch"
 
 
 # The layer sizes that the benchmark runs (width 2048, 32 heads on 4 groups of size 64, feed-forward

@@ -98,9 +98,33 @@ def command_logits(args) -> int:
     return 0
 
 
+class _Range:
+    """A named range for the profiler's timeline (roctx, through torch's marker calls), as the
+    reference marks warmup / prefill / decode with NVTX ranges (app/cuda_reference.cu:31-37)."""
+
+    def __init__(self, name: str):
+        self.name = name
+
+    def __enter__(self):
+        import torch
+        try:
+            torch.cuda.nvtx.range_push(self.name)
+            self.pushed = True
+        except Exception:                      # (a build of torch without the marker library)
+            self.pushed = False
+        return self
+
+    def __exit__(self, *unused):
+        import torch
+        if self.pushed:
+            torch.cuda.nvtx.range_pop()
+        return False
+
+
 def command_benchmark(args) -> int:
     """One request: CONTEXT prompt tokens, OUTPUT_TOKENS greedy tokens; WARMUP runs, then SAMPLES
-    timed ones; medians, as app/cuda_reference.cu:256-471 reports them."""
+    timed ones; medians, the samples, and the device memory's accounting, as
+    app/cuda_reference.cu:256-471 reports them (its keys where it has them)."""
     import statistics
     import torch
     from .engine import StepEntry
@@ -108,33 +132,58 @@ def command_benchmark(args) -> int:
     output_tokens = parse_integer(args.rest[1], "OUTPUT_TOKENS", 1)
     warmup = parse_integer(args.rest[2], "WARMUP", 0)
     samples = parse_integer(args.rest[3], "SAMPLES", 1)
+    if not torch.cuda.is_available():
+        raise EngineError(ErrorCode.HIP, "no GPU is visible: the engine has no CPU path")
+    before_model = torch.cuda.memory_allocated()
     engine = _engine(args, context + output_tokens)
+    model_bytes = torch.cuda.memory_allocated() - before_model
+    cache_bytes = sum(binding.cache.numel() * binding.cache.element_size()
+                      for binding in {id(b.cache): b for b in engine.cache.bindings if b.cache is not None}.values())
     generator = torch.Generator().manual_seed(args.seed)
     prompt = torch.randint(0, engine.spec.vocab_size, (context,), generator=generator).tolist()
-    ttft, tpot, tokens = [], [], None
+    ttft, tpot, tokens, sample_rows = [], [], None, []
+    segments_before = None
     for run in range(warmup + samples):
-        torch.cuda.synchronize()
-        started = time.perf_counter()
-        engine.admit("bench")
-        logits = engine.step([StepEntry("bench", prompt, [context - 1])])
-        token = int(logits.argmax(-1).item())
-        first = time.perf_counter()
-        generated = [token]
-        for _ in range(output_tokens - 1):
-            logits = engine.step([StepEntry("bench", [token], [0])])
-            token = int(logits.argmax(-1).item())
-            generated.append(token)
-        finished = time.perf_counter()
-        engine.finish("bench")
+        if run == warmup:
+            segments_before = torch.cuda.memory_stats().get("segment.all.allocated", 0)
+        with _Range("warmup" if run < warmup else "sample"):
+            torch.cuda.synchronize()
+            started = time.perf_counter()
+            engine.admit("bench")
+            with _Range("prefill"):
+                logits = engine.step([StepEntry("bench", prompt, [context - 1])])
+                token = int(logits.argmax(-1).item())
+            first = time.perf_counter()
+            generated = [token]
+            with _Range("decode"):
+                for _ in range(output_tokens - 1):
+                    logits = engine.step([StepEntry("bench", [token], [0])])
+                    token = int(logits.argmax(-1).item())
+                    generated.append(token)
+            finished = time.perf_counter()
+            engine.finish("bench")
         if tokens is not None and generated != tokens:
             raise EngineError(ErrorCode.NUMERICAL, "benchmark samples did not produce identical tokens")
         tokens = generated
         if run >= warmup:
             ttft.append((first - started) * 1e3)
+            row = {"ttft_ms": ttft[-1]}
             if output_tokens > 1:
                 tpot.append((finished - first) * 1e3 / (output_tokens - 1))
-    result = {"context": context, "output_tokens": output_tokens, "warmup": warmup, "samples": samples,
-              "dtype": args.dtype, "ttft_ms_median": statistics.median(ttft),
+                row["tpot_ms"] = tpot[-1]
+            sample_rows.append(row)
+    # (the reference fails its benchmark when the timed workload allocates device memory:
+    # app/cuda_reference.cu:412-416; here the numbers of segments the allocator has taken from the
+    # device before and after the samples are reported)
+    segments_after = torch.cuda.memory_stats().get("segment.all.allocated", 0)
+    properties = torch.cuda.get_device_properties(engine.device)
+    result = {"schema_version": 1, "gpu": properties.name, "vram_bytes": properties.total_memory,
+              "model_device_bytes": model_bytes, "engine_peak_device_bytes": torch.cuda.max_memory_allocated(),
+              "device_segments_before_workload": segments_before, "device_segments_after_workload": segments_after,
+              "kv_cache_bytes": cache_bytes, "dtype": args.dtype, "sampling": "greedy", "batch": 1,
+              "context": context, "output_tokens": output_tokens, "warmup": warmup, "sample_count": samples,
+              "samples": sample_rows, "generated_tokens": tokens,
+              "ttft_ms_median": statistics.median(ttft),
               "prefill_tokens_per_second": context / (statistics.median(ttft) / 1e3)}
     if tpot:
         result["tpot_ms_median"] = statistics.median(tpot)
