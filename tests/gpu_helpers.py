@@ -23,14 +23,17 @@ CONFIG_B = dict(model_type="llama", architectures=["LlamaForCausalLM"], hidden_s
 CONFIGS = {"A": CONFIG_A, "B": CONFIG_B}
 DTYPES = ["float32", "bfloat16"]
 
-# Differences from the plain implementation (float64 on the same stored weights), relative to the
-# largest logit of the comparison.  float32: rounding of 32-bit sums over at most a few hundred
-# terms.  bfloat16: activations between kernels are rounded to 8 bits of mantissa (2^-9 relative
-# each); a few dozen such roundings per token pile up to about a percent of the logits' size.
-TOLERANCE = {"float32": 2e-5, "bfloat16": 3e-2}
+# Differences from the plain implementation (float64 on the same stored weights), row by row: a
+# row's largest error relative to the row's largest value (a row of small logits is held to its
+# own size, not to the largest logit of the whole comparison).  float32: rounding of 32-bit sums
+# over at most a few hundred terms.  bfloat16: activations between kernels are rounded to 8 bits of
+# mantissa (2^-9 relative each); a few dozen such roundings per token pile up to about a percent.
+TOLERANCE = {"float32": 2e-5, "bfloat16": 1.5e-2}
 # Two ways of cutting the same request through the same engine differ by less: float32 sums run
-# in the same order whatever the cut; bfloat16 may take another kernel for one token than for many.
-CUT_TOLERANCE = {"float32": 1e-6, "bfloat16": 3e-2}
+# in the same order whatever the cut; bfloat16 may take another kernel for one token than for many
+# (and a step that is replayed from a recording must equal the same step launched kernel by kernel
+# bit for bit: the tests that compare those two use torch.equal, not a tolerance).
+CUT_TOLERANCE = {"float32": 1e-6, "bfloat16": 1.5e-2}
 
 
 def make_model(folder, raw_config, seed, dtype_name, std=0.08, norm_std=0.1):
@@ -56,25 +59,35 @@ def random_tokens(seed, count, vocab):
     return [rng.randrange(vocab) for _ in range(count)]
 
 
-def close(got, want, tolerance):
-    """max |got - want| <= tolerance * max |want|; returns (ok, error, scale)."""
+def _row_errors(got, want):
+    """Per row (everything but the last dimension): the largest error and the largest wanted value."""
     got, want = got.double().cpu(), want.double().cpu()
     assert got.shape == want.shape, (got.shape, want.shape)
-    scale = want.abs().max().item()
-    error = (got - want).abs().max().item()
-    return error <= tolerance * scale, error, scale
+    if got.dim() < 2:
+        got, want = got.reshape(1, -1), want.reshape(1, -1)
+    got, want = got.reshape(-1, got.shape[-1]), want.reshape(-1, want.shape[-1])
+    return (got - want).abs().amax(dim=-1), want.abs().amax(dim=-1)
+
+
+def close(got, want, tolerance):
+    """Every row: max |got - want| <= tolerance * max |want| of that row; returns (ok, the worst
+    row's error, that row's scale)."""
+    errors, scales = _row_errors(got, want)
+    excess = errors - tolerance * scales
+    worst = int(excess.argmax())
+    return bool((excess <= 0).all()), errors[worst].item(), scales[worst].item()
 
 
 def assert_close(got, want, tolerance, what=""):
     ok, error, scale = close(got, want, tolerance)
-    assert ok, f"{what}: max error {error:.3e} against scale {scale:.3e} exceeds {tolerance:.1e} relative"
+    assert ok, f"{what}: a row's max error {error:.3e} against its scale {scale:.3e} exceeds {tolerance:.1e} relative"
 
 
 def first_bad_row(got, want, tolerance):
-    """Index of the first row whose error exceeds the tolerance, for messages."""
-    got, want = got.double().cpu(), want.double().cpu()
-    scale = want.abs().max().item()
-    rows = ((got - want).abs().amax(dim=-1) > tolerance * scale).nonzero().flatten().tolist()
+    """Index of the first row whose error exceeds the tolerance (relative to that row's largest
+    wanted value), for messages."""
+    errors, scales = _row_errors(got, want)
+    rows = (errors > tolerance * scales).nonzero().flatten().tolist()
     return rows[0] if rows else None
 
 

@@ -96,6 +96,32 @@ def test_a_step_reserves_for_all_its_requests_or_for_none():
     assert cache.held("a").serial not in before and cache.held("b").serial == before[1]
 
 
+def test_a_step_that_did_not_run_gives_its_reservation_back():
+    """What a step reserved and then did not run (its launch raised) goes back; the request keeps
+    the pages its committed positions lie on, and the next reservation may get other pages."""
+    cache = manager()                                             # 8 pages of 4 positions
+    cache.admit("a")
+    cache.admit("b")
+    assert cache.reserve_all([("a", 6)])
+    cache.commit("a", 6)                                          # pages 0, 1
+    assert cache.reserve_all([("a", 9), ("b", 3)])                # "a" up to 15 positions: pages 2, 3; "b": page 4
+    assert cache.page_list("a", 0) == [0, 1, 2, 3] and cache.free_pages() == [3]
+    cache.unreserve("a")
+    cache.unreserve("b")
+    assert cache.page_list("a", 0) == [0, 1] and cache.page_list("b", 0) == [] and cache.free_pages() == [6]
+    assert cache.length("a") == 6
+    cache.check()
+    cache.unreserve("a")                                          # nothing spare: nothing happens
+    assert cache.page_list("a", 0) == [0, 1]
+    assert cache.reserve_all([("b", 3), ("a", 2)])                # 1 + 0: the freed pages come back in the order of their release
+    cache.commit("a", 2)
+    assert cache.reserve_all([("a", 1)])
+    assert cache.page_list("a", 0)[:2] == [0, 1] and len(cache.page_list("a", 0)) == 3
+    cache.check()
+    with pytest.raises(EngineError):
+        cache.unreserve("nobody")
+
+
 def test_request_slots_run_out_and_state_starts_at_zero():
     cache = manager(max_requests=2, state=True)
     assert len(cache.state_areas) == 2 and cache.state_areas[0].shape == (2, 5)

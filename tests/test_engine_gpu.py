@@ -12,6 +12,7 @@ import torch
 from gpu_helpers import (CONFIGS, CUT_TOLERANCE, DTYPES, TOLERANCE, Replayer, assert_close, first_bad_row, load_plain,
                          make_model, random_tokens)
 from plain_llama import plain_forward, plain_generate_greedy
+from tlie_amd import ops
 
 pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -39,10 +40,19 @@ def plain_logits(setup, tokens):
     return setup["plain"][key]
 
 
-def new_engine(setup, dtype, max_tokens=512, page_size=16, max_requests=4, use_graphs=True):
+def new_engine(setup, dtype, max_tokens=512, page_size=16, max_requests=4, use_graphs=True, capture_graphs=True):
     from tlie_amd import Engine
     return Engine(setup["folder"], dtype=dtype, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests,
-                  use_graphs=use_graphs)
+                  use_graphs=use_graphs, capture_graphs=capture_graphs)
+
+
+def assert_same_bits(replayed, launched, what):
+    """A step replayed from a recording runs the same kernels on the same arrays as the same step,
+    padded alike, launched kernel by kernel: the logits must be equal bit for bit (a tolerance
+    would let a stale row of a block table or a padding row that leaks pass)."""
+    assert set(replayed.rows) == set(launched.rows)
+    for key in sorted(replayed.rows, key=str):
+        assert torch.equal(replayed.rows[key], launched.rows[key]), f"{what}: the replayed row {key} differs in bits from the launched one"
 
 
 def request_tokens(name, index, length):
@@ -270,10 +280,11 @@ def test_recorded_portion_steps_replay_like_eager_ones(setups, name, dtype):
     setup = setups(name, dtype)
     recorded, eager = new_engine(setup, dtype, max_tokens=1024, max_requests=8), \
         new_engine(setup, dtype, max_tokens=1024, max_requests=8, use_graphs=False)
+    padded = new_engine(setup, dtype, max_tokens=1024, max_requests=8, capture_graphs=False)
     rng = random.Random(5)
     streams = {f"p{i}": request_tokens(name, 40 + i, n) for i, n in enumerate((97, 64, 31, 120))}
     done = {request: 0 for request in streams}
-    a, b = Replayer(recorded), Replayer(eager)
+    a, b, c = Replayer(recorded), Replayer(eager), Replayer(padded)
     turn = 0
     while any(done[request] < len(tokens) for request, tokens in streams.items()):
         items = []
@@ -287,16 +298,18 @@ def test_recorded_portion_steps_replay_like_eager_ones(setups, name, dtype):
         if not items:
             turn += 1
             continue
-        for replay in (a, b):
+        for replay in (a, b, c):
             replay.step(items)
         if turn % 4 == 2:
             torch.cuda.synchronize()
             extra = request_tokens(name, 300 + turn, 9)
-            for replay in (a, b):                         # an eager step in between: every row wanted
+            for replay in (a, b, c):                      # an eager step in between: every row wanted
                 replay.step([(f"x{turn}", extra, list(range(9)))], end=[f"x{turn}"])
         turn += 1
     graphs = recorded.runner._portion_graphs
     assert len(graphs) >= 2 and all(graph.graph is not None for graph in graphs.values()) and not eager.runner._portion_graphs
+    assert padded.runner._portion_graphs and all(graph.graph is None for graph in padded.runner._portion_graphs.values())
+    assert_same_bits(a, c, "steps of prompt portions")
     assert set(a.rows) == set(b.rows) and len(a.rows) > 30
     keys = sorted(a.rows, key=str)
     got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
@@ -318,27 +331,28 @@ def test_recorded_decode_steps_replay_like_eager_ones(setups, name, dtype):
     setup = setups(name, dtype)
     recorded, eager = new_engine(setup, dtype, max_tokens=1024, max_requests=8), \
         new_engine(setup, dtype, max_tokens=1024, max_requests=8, use_graphs=False)
+    padded = new_engine(setup, dtype, max_tokens=1024, max_requests=8, capture_graphs=False)
     assert recorded.runner.use_graphs and not eager.runner.use_graphs
     prompts = {f"g{i}": request_tokens(name, 70 + i, n) for i, n in enumerate((9, 33, 20))}
     follow = {request: request_tokens(name, 80 + i, 40) for i, request in enumerate(prompts)}
-    a, b = Replayer(recorded), Replayer(eager)
-    for replay in (a, b):
+    a, b, c = Replayer(recorded), Replayer(eager), Replayer(padded)
+    for replay in (a, b, c):
         replay.step([(request, tokens, [len(tokens) - 1]) for request, tokens in prompts.items()])
     live = list(prompts)
     for turn in range(24):
         if turn == 9:
-            for replay in (a, b):                         # a prompt step between replays
+            for replay in (a, b, c):                      # a prompt step between replays
                 replay.step([("late", follow["g0"][:13], [12])])
             live.append("late")
             follow["late"] = request_tokens(name, 90, 40)
         if turn == 15:
-            for replay in (a, b):
+            for replay in (a, b, c):
                 replay.engine.finish("g1")
             live.remove("g1")
         if turn == 19:
             # a request ends and one of the same name, shorter, takes the same row of the recorded step:
             # nothing of the first one's block table may serve the second
-            for replay in (a, b):
+            for replay in (a, b, c):
                 replay.engine.finish("late")
                 for key in [key for key in replay.rows if key[0] == "late"]:
                     replay.rows[("late before", key[1])] = replay.rows.pop(key)
@@ -347,8 +361,11 @@ def test_recorded_decode_steps_replay_like_eager_ones(setups, name, dtype):
         items = [(request, [follow[request][turn]], [0]) for request in live]
         a.step(items)
         b.step(items)
+        c.step(items)
         torch.cuda.synchronize()
     assert recorded.runner._graphs and all(graph.graph is not None for graph in recorded.runner._graphs.values())
+    assert padded.runner._graphs and all(graph.graph is None for graph in padded.runner._graphs.values())
+    assert_same_bits(a, c, "decode steps")
     assert set(a.rows) == set(b.rows)
     keys = sorted(a.rows, key=str)
     got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
@@ -665,24 +682,27 @@ def test_recorded_steps_of_many_requests_replay_like_eager_ones(setups, dtype, m
     setup = setups("B", dtype)
     recorded, eager = new_engine(setup, dtype, max_tokens=4096, max_requests=many), \
         new_engine(setup, dtype, max_tokens=4096, max_requests=many, use_graphs=False)
+    padded = new_engine(setup, dtype, max_tokens=4096, max_requests=many, capture_graphs=False)
     prompts = {f"m{i}": request_tokens("B", 300 + i, 3 + (7 * i) % 23) for i in range(many)}
     follow = {request: request_tokens("B", 400 + i, 12) for i, request in enumerate(prompts)}
-    a, b = Replayer(recorded), Replayer(eager)
-    for replay in (a, b):
+    a, b, c = Replayer(recorded), Replayer(eager), Replayer(padded)
+    for replay in (a, b, c):
         replay.step([(request, tokens, [len(tokens) - 1]) for request, tokens in prompts.items()])
     live = list(prompts)
     for turn in range(12):
         if turn in (4, 8):
             for request in live[5:8]:
-                for replay in (a, b):
+                for replay in (a, b, c):
                     replay.engine.finish(request)
             del live[5:8]
         items = [(request, [follow[request][turn]], [0]) for request in live]
         a.step(items)
         b.step(items)
+        c.step(items)
         torch.cuda.synchronize()
     bucket = 32 if many == 24 else 128
     assert (bucket, 256) in recorded.runner._graphs and recorded.runner._graphs[(bucket, 256)].graph is not None
+    assert_same_bits(a, c, f"decode steps of up to {many} requests")
     keys = sorted(a.rows, key=str)
     assert keys == sorted(b.rows, key=str)
     got, want = torch.stack([a.rows[key] for key in keys]), torch.stack([b.rows[key] for key in keys])
@@ -744,7 +764,7 @@ def test_long_prompts_take_the_walk_through_lds(tmp_path):
     # the step's policy did choose that walk
     engine.admit("check")
     engine.cache.reserve("check", 1700)
-    policy = engine.runner.build_context([StepEntry("check", tokens[:1700], [])]).attention_tiles(2, 2, 16)
+    policy = ops.attention_plan(engine.runner.build_context([StepEntry("check", tokens[:1700], [])]), 2, 2, 16)
     assert policy[5] is True and policy[4] == 4
     engine.finish("check")
 
@@ -769,3 +789,61 @@ def test_decoding_across_the_lengths_that_recordings_are_made_for(tmp_path, dtyp
     assert sorted(engine.runner._graphs) == [(1, 256), (1, 512), (1, 600)]
     bad = first_bad_row(replay.logits_of("r", range(239, 531)), want[239:], TOLERANCE[dtype])
     assert bad is None, f"first wrong position {239 + bad}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_logits_that_are_not_finite_end_generation_and_leave_the_engine_usable(tmp_path, dtype):
+    """A model whose final norm's weight is so large that the logits overflow: sampling marks the
+    row (-1), the decode step that is launched before the host has read that mark takes token 0 and
+    not a row before the embedding table, `generate` raises numerical_error, and everything the
+    call's requests held has come back: the same engine takes the next call (which fails the same
+    way, not with "already live"), and a step with the finiteness check raises too."""
+    from safetensors.torch import load_file, save_file
+    from tlie_amd import Engine, EngineError, ErrorCode, StepEntry
+    folder = make_model(tmp_path / "inf", CONFIGS["A"], seed=3, dtype_name="float32")
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    tensors["model.norm.weight"] = torch.full_like(tensors["model.norm.weight"], 3.0e38)
+    save_file(tensors, path)
+    engine = Engine(folder, dtype=dtype, max_tokens=256, page_size=16, max_requests=4)
+    for _ in range(2):
+        with pytest.raises(EngineError) as caught:
+            engine.generate([[1, 2, 3], [4, 5, 6, 7]], max_tokens=6)
+        assert caught.value.code == ErrorCode.NUMERICAL
+        engine.cache.check()
+        assert engine.cache.live_requests() == [] and engine.cache.free_pages() == [engine.cache.num_pages]
+    engine.admit("s")
+    logits = engine.step([StepEntry("s", [1, 2, 3], [2])])
+    assert not torch.isfinite(logits).all()
+    with pytest.raises(EngineError) as caught:
+        engine.step([StepEntry("s", [4], [0])], check_finite=True)
+    assert caught.value.code == ErrorCode.NUMERICAL
+    engine.finish("s")
+    engine.cache.check()
+
+
+def test_a_step_that_fails_after_reserving_gives_its_pages_back(setups):
+    """A step whose launch raises after its pages were reserved (here: a token that is still on
+    the device offered to a step that no recording serves) leaves the cache as it found it, and the
+    next steps of the same requests get right logits."""
+    from tlie_amd import EngineError, StepEntry
+    setup = setups("A", "bfloat16")
+    engine = new_engine(setup, "bfloat16", max_tokens=256)
+    tokens = request_tokens("A", 5, 40)
+    replay = Replayer(engine)
+    replay.step([("r", tokens[:15], [14])])
+    replay.step([("r", tokens[15:16], [0])])                 # a recorded decode step: its rows remember the page list
+    free = engine.cache.free_pages()
+    pages = list(engine.cache.page_list("r", 0))
+    with pytest.raises(EngineError):
+        engine.step([StepEntry("r", tokens[16:17], [], source=0)])     # position 16 lies on a second page: reserved, then refused
+    assert engine.cache.free_pages() == free and engine.cache.page_list("r", 0) == pages and engine.cache.length("r") == 16
+    engine.cache.check()
+    engine.admit("other")                                    # takes the page the failed step had reserved first
+    engine.step([StepEntry("other", tokens[:20], [])])
+    for position in range(16, 40):
+        replay.step([("r", tokens[position:position + 1], [0])])
+    engine.finish("other")
+    engine.finish("r")
+    got = replay.logits_of("r", [14] + list(range(15, 40)))
+    assert first_bad_row(got, plain_logits(setup, tokens)[14:], TOLERANCE["bfloat16"]) is None

@@ -12,6 +12,7 @@ import torch
 
 from plain_llama import plain_attention, plain_linear, plain_rms_norm, plain_rope, plain_silu_mul
 from gpu_helpers import assert_close, load_plain
+from tlie_amd import ops
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -201,8 +202,8 @@ def test_pre_norm_block_part(dtype, rows):
     cache = CacheManager([RunNeed(0, block.mixer.cache_need(), block.mixer.state_need())], 16, 8, 2, DT[dtype], DEV)
     cache.admit("r")
     cache.reserve("r", rows)
-    ctx = build_context(cache, [StepEntry("r", [0] * rows, [])], DEV, few_rows_dtype=DT[dtype])
-    assert ctx.few_rows == (rows <= 16 and dtype == "bfloat16")
+    ctx = build_context(cache, [StepEntry("r", [0] * rows, [])], DEV)
+    assert ops.few_rows_route(rows, DT[dtype]) == (rows <= 16 and dtype == "bfloat16")
     x = torch.randn(rows, 72)
     residual = x.clone().to(DEV)
     pending = block.forward(residual, None, ctx, cache.bindings[0])
@@ -563,3 +564,61 @@ def test_an_embedding_with_learned_positions(tmp_path):
         replay.step([("cut", tokens[place:place + 1], [0])])
     engine.finish("cut")
     assert_close(replay.logits_of("cut", range(70)), want, 2e-5, "in portions and token by token")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_architecture_whose_checkpoint_names_every_place_otherwise(tmp_path, dtype):
+    """The seven places a checkpoint's names come from (the embedding's table, the final norm, the
+    head, and per layer the two norms, the mixer and the feed-forward) are the specification's: an
+    architecture registered here, whose files call all of them otherwise, is written, loaded and
+    stepped with no file of the package changed, and gives the logits of the plain implementation on
+    the same values under the reference's names."""
+    import dataclasses
+    from tlie_amd import Engine, LlamaConfig, write_random_model
+    from tlie_amd.registry import register
+    from plain_llama import plain_forward
+    from gpu_helpers import CONFIG_B, TOLERANCE, Replayer
+
+    @register("architecture", "RenamedForCausalLM")
+    class RenamedConfig(LlamaConfig):
+        @classmethod
+        def from_dict(cls, raw):
+            return super().from_dict({**raw, "architectures": ["LlamaForCausalLM"]})
+
+        def to_dict(self):
+            return {**super().to_dict(), "architectures": ["RenamedForCausalLM"]}
+
+        def to_spec(self):
+            spec = super().to_spec()
+            layers = tuple(dataclasses.replace(layer, prefix=f"h.{index}.", mixer_norm_place="ln_1.", mixer_place="attn.",
+                                               feed_forward_norm_place="ln_2.", feed_forward_place="ffn.")
+                           for index, layer in enumerate(spec.layers))
+            head = dataclasses.replace(spec.head, params={**spec.head.params, "tied_to": "wte.weight"})
+            return dataclasses.replace(spec, layers=layers, head=head, embedding_name="wte.weight", final_norm_prefix="ln_f.",
+                                       head_name="out.weight")
+
+    for tied in (True, False):
+        folder = tmp_path / f"tied{tied}"
+        raw = {**CONFIG_B, "tie_word_embeddings": tied}
+        write_random_model(str(folder), RenamedConfig.from_dict(raw), seed=11, std=0.08, norm_std=0.1,
+                           dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+        stored, weights = load_plain(str(folder))
+        assert stored["architectures"] == ["RenamedForCausalLM"]
+        assert "wte.weight" in weights and "ln_f.weight" in weights and "h.0.attn.q_proj.weight" in weights
+        assert ("out.weight" in weights) != tied and not any(name.startswith("model.") for name in weights)
+
+        def reference_name(name):
+            for old, new in (("wte.", "model.embed_tokens."), ("ln_f.", "model.norm."), ("out.", "lm_head."), ("h.", "model.layers."),
+                             (".ln_1.", ".input_layernorm."), (".ln_2.", ".post_attention_layernorm."), (".attn.", ".self_attn."),
+                             (".ffn.", ".mlp.")):
+                name = name.replace(old, new) if old.startswith(".") or name.startswith(old) else name
+            return name
+        tokens = [(29 * i * i + 5) % raw["vocab_size"] for i in range(40)]
+        want = plain_forward(raw, {reference_name(name): tensor for name, tensor in weights.items()}, tokens)
+        engine = Engine(str(folder), dtype=dtype, max_tokens=128, page_size=16, max_requests=2)
+        replay = Replayer(engine)
+        replay.step([("r", tokens[:30], list(range(30)))])
+        for place in range(30, 40):
+            replay.step([("r", tokens[place:place + 1], [0])])
+        assert_close(replay.logits_of("r", range(40)), want, TOLERANCE[dtype], f"renamed checkpoint, tied {tied}")

@@ -134,6 +134,40 @@ def test_pages_run_out_while_decoding_the_last_admitted_is_preempted():
     assert cache.free_pages() == [6] and cache.free_slots == 4
 
 
+def test_a_preempted_request_returns_its_tokens_to_the_steps_budget():
+    """Three decoding requests under a budget of 3 tokens, the last admitted also the first in this
+    step's rotation: when the second one finds no page and preempts it, the token it had in the plan is
+    free again, so the step still takes the other two (the budget is not charged for a request that
+    left the plan)."""
+    cache, scheduler = make(num_pages=6, page_size=4, max_tokens_per_step=3)
+    requests = [Request(name, list(range(base, base + 7)), SamplingParams(max_tokens=8))
+                for name, base in (("a", 1), ("b", 11), ("c", 21))]
+    for request in requests:
+        scheduler.add(request)
+    log = []
+    drive(cache, scheduler, log)
+    for request in requests:
+        assert request.generated == expected_output(request.prompt, 8)
+    assert scheduler.stats["preemptions"] >= 1
+    # in the step that preempted, what was planned never exceeded the budget, and no step of
+    # several decoding requests shrank to fewer tokens than the requests that stayed could use
+    for step in log:
+        assert sum(count for (_, _, count, _) in step) <= 3
+    assert cache.free_pages() == [6] and cache.free_slots == 4
+
+
+def test_budget_after_preemption_is_what_the_plan_holds():
+    """Directly: the tokens of an item that preemption takes out of the plan are handed back."""
+    cache, scheduler = make(num_pages=8, page_size=4)
+    a = Request("a", [1, 2, 3], SamplingParams(max_tokens=4))
+    scheduler.add(a)
+    plan = scheduler.schedule()
+    assert [(item.request.id, item.count) for item in plan] == [("a", 3)]
+    planned = [cache.pages_needed("a", 3)[0]]
+    assert scheduler._preempt(a, plan, planned) == 3 and plan == [] and planned == [0]
+    assert a.state == "waiting" and not cache.is_live("a")
+
+
 def test_prompts_that_block_each_other_are_untangled():
     # two prompts of 28 tokens (7 pages each) in a pool of 10: cut into portions of 8 they take
     # pages turn by turn until neither can go on; the later one is preempted, the earlier finishes.

@@ -204,6 +204,18 @@ class CacheManager:
             entry.pages[group].extend(self.groups[group].allocator.alloc(more))
         return True
 
+    def unreserve(self, request: Hashable) -> None:
+        """Gives back the pages the request holds beyond those its committed length lies on: what a
+        step reserved and then did not run."""
+        entry = self._entry(request)
+        keep = self._blocks_for(entry.length)
+        for group_index, group in enumerate(self.groups):
+            pages = entry.pages[group_index]
+            spare = [page for page in pages[keep:] if page != ABSENT]
+            if spare:
+                group.allocator.release(spare)
+            del pages[keep:]
+
     def commit(self, request: Hashable, count: int) -> None:
         """The step that wrote `count` more positions is enqueued: the request is that much
         longer; a windowed group gives back pages that no later token can see."""

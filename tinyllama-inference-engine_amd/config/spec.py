@@ -25,13 +25,19 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer's parts and the prefix its tensors are stored under."""
+    """One layer's parts, the prefix its tensors are stored under, and under that prefix the place
+    of each part's tensors (the defaults are the names of the reference's checkpoints,
+    src/model_config.cpp:81-95; an architecture whose files name them otherwise says so here)."""
     prefix: str                 # e.g. "model.layers.3."
     block: str                  # arrangement of the parts, e.g. "pre_norm"
     mixer: PartSpec
     feed_forward: PartSpec
     mixer_norm: PartSpec        # the norm in front of the mixer
     feed_forward_norm: PartSpec  # the norm in front of the feed-forward
+    mixer_norm_place: str = "input_layernorm."
+    mixer_place: str = "self_attn."
+    feed_forward_norm_place: str = "post_attention_layernorm."
+    feed_forward_place: str = "mlp."
 
 
 @dataclass(frozen=True)
@@ -60,6 +66,11 @@ class ModelSpec:
     head: PartSpec
     bos_token_id: int = -1
     eos_token_id: int = -1
+    # where the checkpoint keeps what stands outside the layers (the reference's names,
+    # src/model_config.cpp:79,96-97): the embedding's table, the final norm's prefix, the head's matrix
+    embedding_name: str = "model.embed_tokens.weight"
+    final_norm_prefix: str = "model.norm."
+    head_name: str = "lm_head.weight"
 
     def validate(self) -> None:
         from ..errors import invalid_config

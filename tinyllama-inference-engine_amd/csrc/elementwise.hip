@@ -156,6 +156,17 @@ __global__ void silu_mul_wide_kernel(const D* __restrict__ gate_up, int nsplit, 
   }
 }
 
+// ---- out[r, c] = product[r, c] + bias[c] ------------------------------------------------------
+// For a product that a library made without its bias (steps of many rows): the bias joins the
+// float sums, as in the kernels that add it themselves, and the result is rounded once.
+// reference: AddBiasKernel after the library's product (src/cuda/kernels.cu:198-206).
+template <typename B, typename O>
+__global__ void add_bias_kernel(const float* __restrict__ product, const B* __restrict__ bias, O* __restrict__ out,
+                                size_t total, int cols) {
+  for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total; i += static_cast<size_t>(gridDim.x) * blockDim.x)
+    out[i] = from_float<O>(product[i] + to_float(bias[i % cols]));
+}
+
 }  // namespace tlie
 
 using namespace tlie;
@@ -254,4 +265,26 @@ extern "C" int tlie_silu_mul(const void* gate_up, int in_dtype, int nsplit, long
   else
     return kBadArgument;
   return launch_status();
+}
+
+// product float [rows, cols], bias [cols] (float or bfloat16), out [rows, cols] (float: may be `product` itself; or bfloat16).
+extern "C" int tlie_add_bias(const float* product, const void* bias, int bias_dtype, void* out, int out_dtype, int rows,
+                             int cols, void* stream) {
+  if (rows <= 0 || cols <= 0) return kBadArgument;
+  const size_t total = static_cast<size_t>(rows) * cols;
+  const int threads = 256;
+  const int blocks = static_cast<int>((total + threads - 1) / threads < 16384 ? (total + threads - 1) / threads : 16384);
+  hipStream_t s = (hipStream_t)stream;
+#define TLIE_CASE(BC, B, OC, O)                                                                                  \
+  if (bias_dtype == BC && out_dtype == OC) {                                                                     \
+    hipLaunchKernelGGL((add_bias_kernel<B, O>), dim3(blocks), dim3(threads), 0, s, product, (const B*)bias, (O*)out, \
+                       total, cols);                                                                             \
+    return launch_status();                                                                                      \
+  }
+  TLIE_CASE(kF32, float, kF32, float)
+  TLIE_CASE(kF32, float, kBF16, bf16)
+  TLIE_CASE(kBF16, bf16, kF32, float)
+  TLIE_CASE(kBF16, bf16, kBF16, bf16)
+#undef TLIE_CASE
+  return kBadArgument;
 }

@@ -163,17 +163,20 @@ using namespace tlie;
 
 // temperature, top_p, seed, counter: arrays of `rows` entries, or null (greedy for every row).
 // tokens[i] = sampled[source[i]] where source[i] >= 0: a decode step whose tokens are the last step's
-// samples takes them on the device, before the host has read them.
+// samples takes them on the device, before the host has read them.  A sample of -1 (the row's logits
+// held a NaN or an infinity; the host raises numerical_error when it reads it) becomes token 0 here,
+// and a value beyond the vocabulary is clamped to its last entry: the step that is already on its way
+// must not index the embedding table outside its rows.
 __global__ void feed_tokens_kernel(int* __restrict__ tokens, const int* __restrict__ source,
-                                   const int* __restrict__ sampled, int count) {
+                                   const int* __restrict__ sampled, int count, int vocab) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < count && source[i] >= 0) tokens[i] = sampled[source[i]];
+  if (i < count && source[i] >= 0) tokens[i] = min(max(sampled[source[i]], 0), vocab - 1);
 }
 
-extern "C" int tlie_feed_tokens(int* tokens, const int* source, const int* sampled, int count, void* stream) {
-  if (count <= 0) return kBadArgument;
+extern "C" int tlie_feed_tokens(int* tokens, const int* source, const int* sampled, int count, int vocab, void* stream) {
+  if (count <= 0 || vocab <= 0) return kBadArgument;
   hipLaunchKernelGGL(feed_tokens_kernel, dim3((count + 63) / 64), dim3(64), 0, (hipStream_t)stream, tokens, source,
-                     sampled, count);
+                     sampled, count, vocab);
   return launch_status();
 }
 

@@ -39,13 +39,16 @@ def parse_dtype(name) -> torch.dtype:
 class Engine:
     def __init__(self, model_dir: str | None, dtype="bfloat16", max_tokens: int = 4096, page_size: int = 16,
                  max_requests: int = 64, device: str = "cuda:0", config: dict | None = None,
-                 random_seed: int | None = None, use_graphs: bool = True, expect_sha256: str | None = None):
+                 random_seed: int | None = None, use_graphs: bool = True, expect_sha256: str | None = None,
+                 capture_graphs: bool = True):
         """max_tokens: how many positions the cache pools hold in all (rounded up to whole
         pages); max_requests: how many requests can be live at once.
 
         Without a folder, `config` (the contents of a config.json) and `random_seed` give a model
         of random weights drawn on the device, with no file in between (for measurements).
-        expect_sha256: the digest the folder's weight file must have (`checksum_mismatch` otherwise)."""
+        expect_sha256: the digest the folder's weight file must have (`checksum_mismatch` otherwise).
+        use_graphs=False: no step is recorded or padded to a recording's size.  capture_graphs=False:
+        steps are padded and laid out as for a recording but launched kernel by kernel (for checks)."""
         if not torch.cuda.is_available():
             raise EngineError(ErrorCode.HIP, "no GPU is visible: the engine has no CPU path")
         self.dtype = parse_dtype(dtype)
@@ -75,7 +78,7 @@ class Engine:
         with device_memory_errors(f"cache pools of {num_pages} pages"):
             self.cache = CacheManager(self.model.run_needs(), page_size, num_pages, max_requests, self.dtype, self.device,
                                       max_positions=self.spec.max_positions)
-        self.runner = ModelRunner(self.model, self.cache, use_graphs=use_graphs)
+        self.runner = ModelRunner(self.model, self.cache, use_graphs=use_graphs, capture=capture_graphs)
         self.sampler = Sampler(self.device, capacity=max(max_requests, 1))
         self.runner.device_tokens = self.sampler.device_tokens
         self.stats = {"steps": 0, "steps_ahead": 0}      # steps run by `run`; those whose tokens were read a step later
@@ -87,11 +90,21 @@ class Engine:
     def finish(self, request: Hashable) -> None:
         self.cache.release(request)
 
-    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, trace: dict | None = None) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, trace: dict | None = None,
+             check_finite: bool = False) -> torch.Tensor:
         """One step of the model: see `ModelRunner.step`.  The logits are the caller's own (those
         of a step replayed from a recording are copied out of the recording's memory).  `trace`: a
-        dict that receives the step's intermediate tensors by the names of the reference's ModelTrace."""
-        return self.runner.step(entries, timings, trace=trace)
+        dict that receives the step's intermediate tensors by the names of the reference's ModelTrace.
+        check_finite: a NaN or an infinity among the logits is `numerical_error`, as the reference
+        checks what it returns (src/cuda/model.cu:505-510); the step then waits for the device (the
+        sampling kernel's test of a row runs over the logits and its marks are read)."""
+        logits = self.runner.step(entries, timings, trace=trace)
+        if check_finite and logits.shape[0] > 0:
+            from ..ops import sample
+            marks = sample(logits)
+            if int(marks.min().item()) < 0:
+                raise EngineError(ErrorCode.NUMERICAL, "the step's logits hold a NaN or an infinity")
+        return logits
 
     # ---- generation -------------------------------------------------------------------------------
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,
@@ -113,7 +126,15 @@ class Engine:
             request = Request(id=("generate", index), prompt=[int(token) for token in prompt], params=params)
             scheduler.add(request)
             requests.append(request)
-        self.run(scheduler, timings)
+        try:
+            self.run(scheduler, timings)
+        except BaseException:
+            # a step raised (no request can move, a NaN in the logits, a device error): what this
+            # call's requests hold goes back, so that the engine can be used again
+            for request in requests:
+                if self.cache.is_live(request.id):
+                    self.cache.release(request.id)
+            raise
         return [request.generated for request in requests]
 
     def run(self, scheduler: Scheduler, timings: dict | None = None, max_steps: int | None = None) -> int:
@@ -172,12 +193,22 @@ class Engine:
                     self.stats["steps_ahead"] += 1
                 else:
                     scheduler.update(plan, pending.read())
-        finally:
+        except BaseException:
             if behind is not None:
-                # also when a step raised: the requests get the tokens that were sampled for them
+                # the requests get the tokens that were sampled for them before the step that raised;
+                # what reading them raises in turn (a NaN in that step's logits, say) must not
+                # take the place of the error already on its way
                 plan, pending, _ = behind
                 behind = None
-                scheduler.resolve(plan, pending.read())
+                try:
+                    scheduler.resolve(plan, pending.read())
+                except Exception:
+                    pass
+            raise
+        if behind is not None:
+            plan, pending, _ = behind
+            behind = None
+            scheduler.resolve(plan, pending.read())
         return steps
 
     def _device_sources(self, plan, behind):

@@ -197,7 +197,7 @@ class Scheduler:
                 victim = max(self.running, key=lambda candidate: candidate.order)
                 if victim is request and len(self.running) == 1:
                     raise out_of_memory(f"request {request.id!r} does not fit the pool alone")   # add() rules this out
-                self._preempt(victim, plan, planned_pages)
+                budget += self._preempt(victim, plan, planned_pages)     # what the victim had planned is free for others
                 planned.discard(victim.id)
             if request.state == "running":
                 take(request, 1, needed)
@@ -242,7 +242,10 @@ class Scheduler:
             room = min(room, (held + free - planned_pages[group]) * page_size - length)
         return max(0, min(count, room))
 
-    def _preempt(self, victim: Request, plan: list[Scheduled], planned_pages: list[int]) -> None:
+    def _preempt(self, victim: Request, plan: list[Scheduled], planned_pages: list[int]) -> int:
+        """Takes the victim out of the plan and out of the cache and puts it back in front of the
+        queue; returns the tokens it had in the plan."""
+        removed = 0
         for item in list(plan):
             if item.request is victim:
                 # its planned pages were counted against free pages that its release now returns
@@ -250,6 +253,7 @@ class Scheduler:
                 for group, need in enumerate(needed):
                     planned_pages[group] -= need
                 plan.remove(item)
+                removed += item.count
         self.cache.release(victim.id)
         self.running.remove(victim)
         victim.state = "waiting"
@@ -257,6 +261,7 @@ class Scheduler:
         victim.preemptions += 1
         self.stats["preemptions"] += 1
         self.waiting.appendleft(victim)
+        return removed
 
     # ---- after the step ----------------------------------------------------------------------------
     def update(self, plan: list[Scheduled], sampled: list[int] | None) -> list[Request]:

@@ -73,87 +73,23 @@ class StepContext:
     want_rows: torch.Tensor        # int32 [num_wanted] token indices
     groups: list[GroupView]
     host: dict                     # the same arrays as numpy, by name
-    few_rows: bool = False         # at most 16 tokens of bfloat16: the step may use the products that fold norms and adds in
     wants_all_rows: bool = False   # the wanted rows are all the step's tokens, in order
     compute_units: int = 256       # of the device: how many workgroups start at once
-    # a recorded step of prompt portions: its work lists live at fixed addresses, at a fixed size
-    # (the recording's owner makes them: `tiles_for(key, list) -> tensor`); None: a list per step
+    # a recorded step of prompt portions: work lists that parts make on the host live at fixed
+    # addresses, at a fixed size (the recording's owner keeps them: `tiles_for(key, list) -> tensor`,
+    # and makes them again for every replay); None: a list per step
     tile_owner: object = None
     # a dict that receives named copies of the step's intermediate tensors (such a step is never
     # replayed from a recording and takes no fused route), and the name's prefix for the layer that runs
     trace: dict | None = None
     trace_prefix: str = ""
-    _tiles: dict = field(default_factory=dict)
-
-    def attention_tiles(self, groups_per_kv: int, num_kv_heads: int, head_dim: int):
-        """The tiled attention kernel's work list for this step (made once per group size; None
-        for a decode step, whose tiles the kernel derives itself), and how the keys are cut: into
-        as many parts as it takes to give a step of few tiles about a thousand waves (measured: at
-        batch 64 and 2048 positions 4 parts reach 5 TB/s, 16 parts 4 TB/s, and merging more than 16
-        costs more than it gains), each part a multiple of 32 positions and at least 64.
-        Returns (tiles, col_tiles, nsplit, split_len, waves, shared): `waves` of a workgroup share a
-        tile's keys, or with `shared` take columns of their own and get the keys through LDS."""
-        from ..ops import attention_max_waves
-        decode = self.max_new == 1 and self.num_seqs == self.num_tokens
-        col_tiles, shared = 1, False
-        if decode:
-            tiles, count = None, self.num_tokens * ((groups_per_kv + 15) // 16)
-        else:
-            from ..ops import attention_col_tiles, attention_tiles
-            col_tiles = attention_col_tiles(head_dim)
-            # sequences of some length with portions of many columns: 4 waves take columns of their own
-            # of one tile and every block of keys is brought once for all of them, through LDS (a
-            # prompt of 1536 tokens: 34 us against 42; of 8192: 500 against 780; of 512: 15 against
-            # 13).  Each wave takes 32 columns, or 16 while that leaves no more tiles than two for
-            # every compute unit: they are then all at work at once, and smaller ones fill the chip
-            # better (1024 tokens: 24 us against 30; from 3072 on the larger tiles win)
-            shared = (col_tiles == 2 and head_dim <= 128 and self.max_context >= 768
-                      and self.num_tokens * groups_per_kv >= 64 * self.num_seqs)
-
-            def tiles_of(groups):
-                if (groups_per_kv, groups) not in self._tiles:
-                    made = attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"])
-                    if self.tile_owner is not None:
-                        self._tiles[(groups_per_kv, groups)] = self.tile_owner.tiles_for((groups_per_kv, groups), made)
-                    else:
-                        self._tiles[(groups_per_kv, groups)] = torch.from_numpy(made).to(self.tokens.device)
-                return self._tiles[(groups_per_kv, groups)]
-            tiles = tiles_of(col_tiles * (4 if shared else 1))
-            if shared and tiles.shape[0] * num_kv_heads <= 2 * self.compute_units:
-                col_tiles = 1
-                tiles = tiles_of(4)
-            count = tiles.shape[0] * (4 if shared else 1)
-        tiles_all = count * num_kv_heads
-        if not decode:
-            # a step of prompt portions has tiles enough; cutting their keys would only add merging.
-            # Up to 4 waves share a tile's keys, each with 128 or more: a tile that sees the whole of
-            # a long sequence then takes a quarter of the time, and it is the longest tiles that
-            # the step waits for (a prompt of 2048 tokens: 70 us against 87 with one wave a tile)
-            nsplit = max(1, min((512 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
-            waves = 4 if shared else 1
-            while (not shared and waves < 4 and waves * 2 <= attention_max_waves(head_dim, col_tiles)
-                   and self.max_context >= nsplit * waves * 2 * 128):
-                waves *= 2
-        else:
-            # workgroups share a tile's keys until there is one for every compute unit (their sums
-            # meet in the merge kernel); then the waves of a workgroup share them, which costs no
-            # launch, while a wave keeps 128 keys or more and the step has 2048 waves at most
-            # (measured inside whole steps at 2048 positions: batch 1 16 parts x 1 wave, batch 8
-            # 8 x 2, batch 64 1 x 8)
-            nsplit = max(1, min((256 + tiles_all - 1) // tiles_all, 16, (self.max_context + 63) // 64))
-            waves = 1
-            while (waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 2048
-                   and self.max_context >= nsplit * waves * 2 * 128):
-                waves *= 2
-        if nsplit == 1:
-            return tiles, col_tiles, 1, 0, waves, shared
-        split_len = ((self.max_context + nsplit - 1) // nsplit + 31) // 32 * 32
-        nsplit = (self.max_context + split_len - 1) // split_len
-        return tiles, col_tiles, nsplit, split_len, waves, shared
+    # what parts keep for the length of this step, under keys of their own (work lists that several
+    # layers share, say); the step function never looks inside
+    scratch: dict = field(default_factory=dict)
 
 
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, use_graphs: bool = True):
+    def __init__(self, model, cache: CacheManager, use_graphs: bool = True, capture: bool = True):
         self.model = model
         self.cache = cache
         self.device = model.device
@@ -164,6 +100,9 @@ class ModelRunner:
         # so is a step of prompt portions per (tokens, sequences, range of lengths) padded up.
         # Parts say whether they may be captured (`graph_safe`).
         self.use_graphs = use_graphs and getattr(model, "graph_safe", False) and torch.device(self.device).type == "cuda"
+        # capture=False: the steps a recording would serve are still padded to its sizes and run on
+        # its fixed arrays, but launched kernel by kernel every time (what a replay must equal bit for bit)
+        self.capture = capture
         self.device_tokens: torch.Tensor | None = None     # int32, where sampling leaves a step's tokens (set by the engine)
         self._graphs: dict[tuple[int, int], "DecodeGraph"] = {}      # by (most sequences, longest sequence)
         self._portion_graphs: dict[tuple[int, int, int], "PortionGraph"] = {}   # by (most tokens, most sequences, longest sequence)
@@ -195,7 +134,7 @@ class ModelRunner:
                 raise out_of_bounds(f"request {entry.request!r} would pass the model's {limit} positions")
 
     def build_context(self, entries: Sequence[StepEntry]) -> StepContext:
-        return build_context(self.cache, entries, self.device, few_rows_dtype=self.model.dtype)
+        return build_context(self.cache, entries, self.device)
 
     def _length_bucket(self, longest: int) -> int:
         """The sequence length a recording is made for: the next power of two from 256 on, up to
@@ -252,38 +191,47 @@ class ModelRunner:
         wanted = [(entry.request, len(entry.tokens)) for entry in entries]
         if not self.cache.reserve_all(wanted):
             raise out_of_memory(f"the step needs more pages than are free ({self.cache.free_pages()} free)")
-        if marks:
-            marks[0].record()
-        if trace is None and self.replays(entries):
-            longest = max(self.cache.length(request) + count for request, count in wanted)
-            key = (DecodeGraph.bucket_of(len(entries)), self._length_bucket(longest))
-            if key not in self._graphs:
-                self._graphs[key] = DecodeGraph(self, *key)
-            logits = self._graphs[key].run(entries, marks[1] if marks else None)
-            if keep:
-                logits = logits.clone()
-        elif trace is None and (sizes := self.records(entries)) is not None:
-            longest = max(self.cache.length(request) + count for request, count in wanted)
-            key = (*sizes, self._length_bucket(longest))
-            if key not in self._portion_graphs:
-                self._portion_graphs[key] = PortionGraph(self, *key)
-            logits = self._portion_graphs[key].run(entries, marks[1] if marks else None)
-            if keep:
-                logits = logits.clone()
-        else:
-            if any(entry.source is not None for entry in entries):
-                raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
-            ctx = self.build_context(entries)
-            ctx.trace = trace
+        try:
             if marks:
-                marks[1].record()
-            logits = self.model.forward(ctx, self.cache.bindings)
-        if marks:
-            marks[2].record()
-            marks[2].synchronize()
-            timings.transfer_ms = marks[0].elapsed_time(marks[1])
-            timings.compute_ms = marks[1].elapsed_time(marks[2])
-            timings.wall_ms = (time.perf_counter() - started) * 1e3
+                marks[0].record()
+            if trace is None and self.replays(entries):
+                longest = max(self.cache.length(request) + count for request, count in wanted)
+                key = (DecodeGraph.bucket_of(len(entries)), self._length_bucket(longest))
+                if key not in self._graphs:
+                    self._graphs[key] = DecodeGraph(self, *key)
+                logits = self._graphs[key].run(entries, marks[1] if marks else None)
+                if keep:
+                    logits = logits.clone()
+            elif trace is None and (sizes := self.records(entries)) is not None:
+                longest = max(self.cache.length(request) + count for request, count in wanted)
+                key = (*sizes, self._length_bucket(longest))
+                if key not in self._portion_graphs:
+                    self._portion_graphs[key] = PortionGraph(self, *key)
+                logits = self._portion_graphs[key].run(entries, marks[1] if marks else None)
+                if keep:
+                    logits = logits.clone()
+            else:
+                if any(entry.source is not None for entry in entries):
+                    raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
+                ctx = self.build_context(entries)
+                ctx.trace = trace
+                if marks:
+                    marks[1].record()
+                logits = self.model.forward(ctx, self.cache.bindings)
+            if marks:
+                marks[2].record()
+                marks[2].synchronize()
+                timings.transfer_ms = marks[0].elapsed_time(marks[1])
+                timings.compute_ms = marks[1].elapsed_time(marks[2])
+                timings.wall_ms = (time.perf_counter() - started) * 1e3
+        except BaseException:
+            # nothing of the step counts: the pages it reserved go back (the requests keep what
+            # their committed positions lie on), so that a later step finds the lists it expects
+            for request, _ in wanted:
+                self.cache.unreserve(request)
+            for recording in (*self._graphs.values(), *self._portion_graphs.values()):
+                recording.forget()                      # (a page list that shrank and grew again is not the list a row remembers)
+            raise
         for request, count in wanted:
             self.cache.commit(request, count)
         return logits
@@ -351,12 +299,17 @@ class DecodeGraph:
             tokens=views["tokens"], positions=views["positions"], token_seq=views["token_seq"], no_slots=views["no_slots"],
             seq_start=views["seq_start"], seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"],
             seq_slot=views["seq_slot"], want_rows=views["want_rows"], groups=groups, host=self.host,
-            few_rows=bucket <= 16 and runner.model.dtype == torch.bfloat16, wants_all_rows=single,
+            wants_all_rows=single,
             compute_units=_compute_units(runner.device), tile_owner=None if single else self)
         self.graph = None
         self.logits = None
         self._rows_filled = bucket                           # rows that may hold a step's values
         self._known = [[(0, 0)] * bucket for _ in cache.groups]   # per group and row: (admission, blocks written)
+
+    def forget(self) -> None:
+        """What the rows of the block tables are known to hold is no longer trusted: the next step
+        writes them whole."""
+        self._known = [[(0, 0)] * self.bucket for _ in self._known]
 
     @property
     def runner(self) -> "ModelRunner":
@@ -425,13 +378,15 @@ class DecodeGraph:
         self.copied.record()
         self.copy_pending = True
         if any(entry.source is not None for entry in entries):
-            ops_feed_tokens(self.ctx.tokens, self.token_source, runner.device_tokens)
+            ops_feed_tokens(self.ctx.tokens, self.token_source, runner.device_tokens, runner.vocab_size)
         if transferred is not None:
             transferred.record()
         if self.graph is None:
             # the first step of this size runs eagerly (its result is used, and it leaves the
             # context's work lists made); the same launches are then recorded for the steps to come
             logits = runner.model.forward(self.ctx, runner.cache.bindings)
+            if not runner.capture:
+                return logits[:wanted]
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # no garbage collection while the capture is open: collecting some dead object that
@@ -467,32 +422,31 @@ class PortionGraph(DecodeGraph):
 
     def __init__(self, runner: "ModelRunner", tokens: int, seqs: int, longest: int):
         super().__init__(runner, tokens, longest, seqs=seqs)
-        self._lists: dict = {}            # (group size, column groups) -> (pinned list, the list on the device)
+        self._lists: dict = {}            # a part's key -> (pinned list, the list on the device, the function that makes it)
 
-    def tiles_for(self, key, made: np.ndarray) -> torch.Tensor:
-        """The attention work list `key` of this recording, at its fixed place, holding `made`."""
+    def tiles_for(self, key, make, capacity: int) -> torch.Tensor:
+        """A part's work list `key` of this recording, at its fixed place.  `make(host)` builds it
+        from the step's host arrays as int32 [n, 4] (it is called now, and again before every
+        replay); `capacity`: the most rows it can have in a step of this recording's size.  Rows
+        beyond the step's are zero."""
         if key not in self._lists:
             if torch.cuda.is_current_stream_capturing():
                 raise invalid_argument("a work list first asked for inside a recording")
-            groups_per_kv, groups = key
-            # a sequence of n tokens has ceil(n * G / (16 * groups)) tiles
-            capacity = (self.bucket * groups_per_kv + 16 * groups - 1) // (16 * groups) + self.seqs
             self._lists[key] = (torch.zeros((capacity, 4), dtype=torch.int32, pin_memory=True),
-                                torch.zeros((capacity, 4), dtype=torch.int32, device=self.device_flat.device))
-        pinned, device = self._lists[key]
+                                torch.zeros((capacity, 4), dtype=torch.int32, device=self.device_flat.device), make)
+        pinned, device, make = self._lists[key]
+        made = make(self.host)
         if made.shape[0] > pinned.shape[0]:
-            raise invalid_argument(f"{made.shape[0]} attention tiles do not fit the recording's {pinned.shape[0]}")
+            raise invalid_argument(f"{made.shape[0]} rows of a work list do not fit the recording's {pinned.shape[0]}")
         host = pinned.numpy()
         host[:made.shape[0]] = made
-        host[made.shape[0]:] = 0                                  # no tokens: the kernel leaves at once
+        host[made.shape[0]:] = 0                                  # (an attention tile without tokens: the kernel leaves at once)
         device.copy_(pinned, non_blocking=True)
         return device
 
     def _send_lists(self) -> None:
-        from ..ops import attention_tiles
-        for (groups_per_kv, groups) in self._lists:
-            self.tiles_for((groups_per_kv, groups),
-                           attention_tiles(self.host["seq_start"], groups_per_kv, groups, self.host["seq_len"]))
+        for key, (_, _, make) in self._lists.items():
+            self.tiles_for(key, make, 0)
 
     def _fill(self, entries: Sequence[StepEntry]) -> int:
         cache, host = self.runner.cache, self.host
@@ -536,7 +490,7 @@ def _compute_units(device) -> int:
     return int(torch.cuda.get_device_properties(device).multi_processor_count)
 
 
-def build_context(cache: CacheManager, entries: Sequence[StepEntry], device, few_rows_dtype=None) -> StepContext:
+def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> StepContext:
     """The step's arrays for entries whose pages are reserved: built on the host, sent in one
     transfer."""
     counts = [len(entry.tokens) for entry in entries]
@@ -586,7 +540,6 @@ def build_context(cache: CacheManager, entries: Sequence[StepEntry], device, few
         token_seq=views["token_seq"], no_slots=views["no_slots"], seq_start=views["seq_start"],
         seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
         want_rows=views["want_rows"], groups=groups, host=host,
-        few_rows=total <= 16 and few_rows_dtype == torch.bfloat16,
         wants_all_rows=bool(want_rows.size == total and np.array_equal(want_rows, np.arange(total))),
         compute_units=_compute_units(device))
 

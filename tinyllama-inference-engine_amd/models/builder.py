@@ -7,6 +7,7 @@ import torch
 from .. import parts as _parts  # noqa: F401  (fills the part registries)
 from ..cache.manager import RunNeed
 from ..config.spec import ModelSpec, TensorSpec
+from .. import ops
 from ..ops import ResidualUpdated
 from ..registry import lookup
 
@@ -15,11 +16,11 @@ def expected_tensors(spec: ModelSpec) -> list[TensorSpec]:
     """Every tensor the model's parts expect, by full name; the list that weights are checked
     against and that random weights are drawn for (the reference's fixed list of 9 per layer + 3
     is `ExpectedTensors`, src/model_config.cpp:78-97)."""
-    specs = list(lookup("embedding", spec.embedding.kind).tensor_specs(spec.embedding, ""))
+    specs = list(lookup("embedding", spec.embedding.kind).tensor_specs(spec.embedding, spec.embedding_name))
     for layer in spec.layers:
         specs += lookup("block", layer.block).tensor_specs(layer)
-    specs += lookup("norm", spec.final_norm.kind).tensor_specs(spec.final_norm, "model.norm.")
-    specs += lookup("head", spec.head.kind).tensor_specs(spec.head, "")
+    specs += lookup("norm", spec.final_norm.kind).tensor_specs(spec.final_norm, spec.final_norm_prefix)
+    specs += lookup("head", spec.head.kind).tensor_specs(spec.head, spec.head_name)
     names = [tensor.name for tensor in specs]
     if len(set(names)) != len(names):
         raise AssertionError("two parts claim the same tensor name")
@@ -40,11 +41,11 @@ class DecoderModel:
         self.head = lookup("head", spec.head.kind)(spec.head, dtype, device)
 
     def load(self, weights: dict[str, torch.Tensor]) -> None:
-        self.embedding.load(weights, "")
+        self.embedding.load(weights, self.spec.embedding_name)
         for block in self.blocks:
             block.load(weights)
-        self.final_norm.load(weights, "model.norm.")
-        self.head.load(weights, "")
+        self.final_norm.load(weights, self.spec.final_norm_prefix)
+        self.head.load(weights, self.spec.head_name)
 
     @property
     def graph_safe(self) -> bool:
@@ -67,24 +68,30 @@ class DecoderModel:
         (src/model.cpp:98-231)."""
         runs = self.spec.runs
         trace = getattr(ctx, "trace", None)
-        first_norm = self.blocks[runs[0].layer].mixer_norm
-        if (ctx.few_rows and trace is None and hasattr(self.embedding, "forward_rows")
-                and first_norm.lazy_params() is not None):
-            residual, normed = self.embedding.forward_rows(ctx.tokens, first_norm.lazy_params())
+        few = ops.few_rows_route(ctx.num_tokens, self.dtype) and trace is None
+
+        def entry_norm(block):
+            # a block may say which norm reads the residual first (its writer can then leave that
+            # norm's inputs); a block that does not is handed a plain residual
+            return block.entry_norm() if hasattr(block, "entry_norm") else None
+        first_norm = entry_norm(self.blocks[runs[0].layer])
+        lazy = first_norm.lazy_params() if first_norm is not None else None
+        if few and hasattr(self.embedding, "forward_rows") and lazy is not None:
+            residual, normed = self.embedding.forward_rows(ctx.tokens, lazy)
             pending = ResidualUpdated(normed)
         else:
             residual, pending = self.embedding.forward(ctx.tokens, ctx), None
         if trace is not None:
             trace["embedding"] = residual.float().clone()
         for index, run in enumerate(runs):
-            next_norm = self.blocks[runs[index + 1].layer].mixer_norm if index + 1 < len(runs) else self.final_norm
+            next_norm = entry_norm(self.blocks[runs[index + 1].layer]) if index + 1 < len(runs) else self.final_norm
             if trace is not None:
                 ctx.trace_prefix = f"layer{index}."
             pending = self.blocks[run.layer].forward(residual, pending, ctx, bindings[index], next_norm=next_norm)
         if ctx.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if ctx.wants_all_rows:
-            lazy = ctx.few_rows and trace is None and self.head.takes_normed_rows(residual.shape[0])
+            lazy = few and self.head.takes_normed_rows(residual.shape[0])
             normed = self.final_norm.add_forward(residual, pending, lazy=lazy)
         else:
             normed = self.final_norm.add_forward(residual, pending, rows=ctx.want_rows)

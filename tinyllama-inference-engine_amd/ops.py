@@ -16,6 +16,7 @@ from .csrc import build as _build
 from .errors import EngineError, ErrorCode, invalid_argument, invalid_shape
 
 F32, BF16 = 0, 1
+ROWS_MAX = 16          # the most rows the products take that fold in the layer's neighbouring arithmetic
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -274,8 +275,8 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
     rows; y in bfloat16, or in float32 (the output head's logits).  The library is called
     directly, with its plan for the shape kept (half the host time of torch.mm, which a step of
     prompt portions calls four times a layer); where that is not possible (the library's file
-    is not beside torch, or it has no algorithm for the shape) torch.mm makes the same product, or,
-    inside a recording, this library's plain kernel."""
+    is not beside torch, or it has no algorithm for the shape) this library's plain kernel makes the
+    product."""
     if out_dtype not in (torch.bfloat16, torch.float32):
         raise EngineError(ErrorCode.INVALID_DTYPE, f"library_mm gives bfloat16 or float32, not {out_dtype}")
     _device_tensor(x, "x", torch.bfloat16)
@@ -301,13 +302,26 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
             return out
         if status != -3:
             _check(status, "library_gemm")
-    if torch.cuda.is_current_stream_capturing():
-        # inside a recording no library call that has not been tried there: torch's product may clear a
-        # workspace with a memset node, which replays wrongly; the plain kernel is slow and safe
-        return gemm_generic(x, weight, None, out_dtype).data
-    if out_dtype == torch.float32:
-        return torch.mm(x.float(), weight.float().t())
-    return torch.mm(x, weight.t())
+    # where the library cannot be called directly (its file is not beside torch, or it has no
+    # algorithm for the shape) this library's plain kernel makes the product: one route, recorded or
+    # not, so that a step gives the same bits replayed and launched (slow, and safe inside a recording,
+    # where a library call that has not been tried may clear a workspace with a memset node)
+    return gemm_generic(x, weight, None, out_dtype).data
+
+
+def add_bias(product: torch.Tensor, bias: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """out = product + bias (one entry per column) for a float32 product that came without its bias;
+    the sum is float32 and rounded once to `out_dtype` (float32: in place)."""
+    _device_tensor(product, "product", torch.float32)
+    _device_tensor(bias, "bias", (torch.float32, torch.bfloat16))
+    if product.dim() != 2 or bias.shape != (product.shape[1],):
+        raise invalid_shape(f"add_bias: product {list(product.shape)} and bias {list(bias.shape)} do not fit")
+    out = product if out_dtype == torch.float32 else torch.empty(product.shape, dtype=out_dtype, device=product.device)
+    if product.shape[0] == 0:
+        return out
+    _check(library().tlie_add_bias(_ptr(product), _ptr(bias), dtype_code(bias.dtype), _ptr(out), dtype_code(out_dtype),
+                                   product.shape[0], product.shape[1], _stream()), "add_bias")
+    return out
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p: torch.Tensor | None = None,
@@ -340,16 +354,21 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor | None = None, top_p:
     return out
 
 
-def feed_tokens(tokens: torch.Tensor, source: torch.Tensor, sampled: torch.Tensor) -> None:
-    """tokens[i] = sampled[source[i]] wherever source[i] >= 0, on the device.  The caller has
-    checked on the host that every such source is a row of `sampled`."""
+def feed_tokens(tokens: torch.Tensor, source: torch.Tensor, sampled: torch.Tensor, vocab: int) -> None:
+    """tokens[i] = sampled[source[i]] wherever source[i] >= 0, on the device, brought into the
+    vocabulary's range 0 .. vocab - 1 (a sample of -1 marks a row of logits that held a NaN or an
+    infinity: the host raises when it reads it, and the step that is already launched takes token 0).
+    The caller has checked on the host that every such source is a row of `sampled`."""
     for name, tensor in (("tokens", tokens), ("source", source), ("sampled", sampled)):
         _device_tensor(tensor, name, torch.int32)
     if tokens.dim() != 1 or source.shape != tokens.shape or sampled.dim() != 1 or sampled.shape[0] == 0:
         raise invalid_shape("feed_tokens takes tokens [T], source [T] and sampled [rows]")
+    if vocab <= 0:
+        raise invalid_argument("feed_tokens: the vocabulary's size must be positive")
     if tokens.shape[0] == 0:
         return
-    _check(library().tlie_feed_tokens(_ptr(tokens), _ptr(source), _ptr(sampled), tokens.shape[0], _stream()), "feed_tokens")
+    _check(library().tlie_feed_tokens(_ptr(tokens), _ptr(source), _ptr(sampled), tokens.shape[0], int(vocab), _stream()),
+           "feed_tokens")
 
 
 # ---- bfloat16 kernels on the matrix cores ---------------------------------------------------------
@@ -435,6 +454,84 @@ def attention_tiles(seq_start, groups_per_kv: int, col_tiles: int = 1, seq_len=N
     return np.ascontiguousarray(rows)
 
 
+def few_rows_route(rows: int, dtype: torch.dtype) -> bool:
+    """Whether a step of `rows` tokens may take the route on which the products of few rows fold in
+    the norm before them and the add (or gate, or rotation) after them: bfloat16, at most 16 rows."""
+    return dtype == torch.bfloat16 and 0 < rows <= ROWS_MAX
+
+
+def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
+    """How the tiled attention kernel is launched for the step `ctx` describes: its work list (made
+    once per step and group size, kept in `ctx.scratch`; None for a decode step, whose tiles the
+    kernel derives itself), and how the keys are cut: into as many parts as it takes to give a step
+    of few tiles about a thousand waves (measured: at batch 64 and 2048 positions 4 parts reach
+    5 TB/s, 16 parts 4 TB/s, and merging more than 16 costs more than it gains), each part a
+    multiple of 32 positions and at least 64.  The policy is this kernel's own and measured on the
+    MI355X; the step's context only supplies the host arrays, the number of compute units, and, in a
+    recorded step, the owner of work lists at fixed addresses.
+    Returns (tiles, col_tiles, nsplit, split_len, waves, shared): `waves` of a workgroup share a
+    tile's keys, or with `shared` take columns of their own and get the keys through LDS."""
+    decode = ctx.max_new == 1 and ctx.num_seqs == ctx.num_tokens
+    col_tiles, shared = 1, False
+    if decode:
+        tiles, count = None, ctx.num_tokens * ((groups_per_kv + 15) // 16)
+    else:
+        col_tiles = attention_col_tiles(head_dim)
+        # sequences of some length with portions of many columns: 4 waves take columns of their own
+        # of one tile and every block of keys is brought once for all of them, through LDS (a
+        # prompt of 1536 tokens: 34 us against 42; of 8192: 500 against 780; of 512: 15 against
+        # 13).  Each wave takes 32 columns, or 16 while that leaves no more tiles than two for
+        # every compute unit: they are then all at work at once, and smaller ones fill the chip
+        # better (1024 tokens: 24 us against 30; from 3072 on the larger tiles win)
+        shared = (col_tiles == 2 and head_dim <= 128 and ctx.max_context >= 768
+                  and ctx.num_tokens * groups_per_kv >= 64 * ctx.num_seqs)
+
+        def tiles_of(groups):
+            key = ("attention_tiles", groups_per_kv, groups)
+            if key not in ctx.scratch:
+                def make(host):
+                    return attention_tiles(host["seq_start"], groups_per_kv, groups, host["seq_len"])
+                if ctx.tile_owner is not None:
+                    # a sequence of n tokens has ceil(n * G / (16 * groups)) tiles
+                    capacity = (ctx.num_tokens * groups_per_kv + 16 * groups - 1) // (16 * groups) + ctx.num_seqs
+                    ctx.scratch[key] = ctx.tile_owner.tiles_for(key, make, capacity)
+                else:
+                    ctx.scratch[key] = torch.from_numpy(make(ctx.host)).to(ctx.tokens.device)
+            return ctx.scratch[key]
+        tiles = tiles_of(col_tiles * (4 if shared else 1))
+        if shared and tiles.shape[0] * num_kv_heads <= 2 * ctx.compute_units:
+            col_tiles = 1
+            tiles = tiles_of(4)
+        count = tiles.shape[0] * (4 if shared else 1)
+    tiles_all = count * num_kv_heads
+    if not decode:
+        # a step of prompt portions has tiles enough; cutting their keys would only add merging.
+        # Up to 4 waves share a tile's keys, each with 128 or more: a tile that sees the whole of
+        # a long sequence then takes a quarter of the time, and it is the longest tiles that
+        # the step waits for (a prompt of 2048 tokens: 70 us against 87 with one wave a tile)
+        nsplit = max(1, min((512 + tiles_all - 1) // tiles_all, 16, (ctx.max_context + 63) // 64))
+        waves = 4 if shared else 1
+        while (not shared and waves < 4 and waves * 2 <= attention_max_waves(head_dim, col_tiles)
+               and ctx.max_context >= nsplit * waves * 2 * 128):
+            waves *= 2
+    else:
+        # workgroups share a tile's keys until there is one for every compute unit (their sums
+        # meet in the merge kernel); then the waves of a workgroup share them, which costs no
+        # launch, while a wave keeps 128 keys or more and the step has 2048 waves at most
+        # (measured inside whole steps at 2048 positions: batch 1 16 parts x 1 wave, batch 8
+        # 8 x 2, batch 64 1 x 8)
+        nsplit = max(1, min((256 + tiles_all - 1) // tiles_all, 16, (ctx.max_context + 63) // 64))
+        waves = 1
+        while (waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 2048
+               and ctx.max_context >= nsplit * waves * 2 * 128):
+            waves *= 2
+    if nsplit == 1:
+        return tiles, col_tiles, 1, 0, waves, shared
+    split_len = ((ctx.max_context + nsplit - 1) // nsplit + 31) // 32 * 32
+    nsplit = (ctx.max_context + split_len - 1) // split_len
+    return tiles, col_tiles, nsplit, split_len, waves, shared
+
+
 def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
     return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= 256 and page_size >= 16
             and page_size & (page_size - 1) == 0)
@@ -505,7 +602,6 @@ def attention_mfma(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tens
 
 
 # ---- at most 16 rows: products with the layer's neighbouring arithmetic folded in --------------------
-ROWS_MAX = 16
 
 
 @dataclass

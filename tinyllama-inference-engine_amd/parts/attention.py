@@ -99,7 +99,7 @@ class Attention(Mixer):
                                self.dtype, paired=self.paired)
         page_size = binding.cache.shape[3] // self.d
         if ops.attention_mfma_takes(self.dtype, self.d, page_size):
-            tiles, col_tiles, nsplit, split_len, waves, shared = ctx.attention_tiles(self.nq // self.nkv, self.nkv, self.d)
+            tiles, col_tiles, nsplit, split_len, waves, shared = ops.attention_plan(ctx, self.nq // self.nkv, self.nkv, self.d)
             attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv,
                                           self.d, self.window, self.scale, nsplit, split_len, col_tiles, waves, shared)
         else:

@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from ..config.spec import LayerSpec
+from .. import ops
 from ..ops import ResidualUpdated, as_product
 from ..registry import lookup, register
 from .base import ResidualTarget
@@ -20,28 +21,36 @@ from .base import ResidualTarget
 class PreNormBlock:
     def __init__(self, layer: LayerSpec, dtype, device):
         self.layer = layer
+        self.dtype = dtype
         self.mixer_norm = lookup("norm", layer.mixer_norm.kind)(layer.mixer_norm, dtype, device)
         self.mixer = lookup("mixer", layer.mixer.kind)(layer.mixer, dtype, device)
         self.feed_forward_norm = lookup("norm", layer.feed_forward_norm.kind)(layer.feed_forward_norm, dtype, device)
         self.feed_forward = lookup("feed_forward", layer.feed_forward.kind)(layer.feed_forward, dtype, device)
 
-    # names under the layer's prefix, as the reference's checkpoints have them
-    # (src/model_config.cpp:81-95)
-    _PLACES = (("mixer_norm", "input_layernorm."), ("mixer", "self_attn."),
-               ("feed_forward_norm", "post_attention_layernorm."), ("feed_forward", "mlp."))
+    _PARTS = ("mixer_norm", "mixer", "feed_forward_norm", "feed_forward")
+
+    @staticmethod
+    def _place(layer: LayerSpec, attribute: str) -> str:
+        """Where a part's tensors lie: the layer's prefix and the place the layer's spec names."""
+        return layer.prefix + getattr(layer, attribute + "_place")
 
     @classmethod
     def tensor_specs(cls, layer: LayerSpec):
         specs = []
-        for attribute, place in cls._PLACES:
+        for attribute in cls._PARTS:
             part_spec = getattr(layer, attribute)
             table = {"mixer_norm": "norm", "feed_forward_norm": "norm"}.get(attribute, attribute)
-            specs += lookup(table, part_spec.kind).tensor_specs(part_spec, layer.prefix + place)
+            specs += lookup(table, part_spec.kind).tensor_specs(part_spec, cls._place(layer, attribute))
         return specs
 
     def load(self, weights):
-        for attribute, place in self._PLACES:
-            getattr(self, attribute).load(weights, self.layer.prefix + place)
+        for attribute in self._PARTS:
+            getattr(self, attribute).load(weights, self._place(self.layer, attribute))
+
+    def entry_norm(self):
+        """The norm that reads the residual first in this block: whoever writes the residual before
+        the block (the embedding, the block before) may leave that norm's inputs with it."""
+        return self.mixer_norm
 
     @property
     def graph_safe(self) -> bool:
@@ -59,7 +68,7 @@ class PreNormBlock:
         if getattr(ctx, "trace", None) is not None:
             return self._forward_traced(residual, pending, ctx, binding)
         rows = residual.shape[0]
-        few = ctx.few_rows
+        few = ops.few_rows_route(rows, self.dtype)
         normed = self.mixer_norm.add_forward(residual, pending, lazy=few and self.mixer.takes_normed_rows(rows))
         if few and self.mixer.adds_to_residual:
             mixed = self.mixer.forward(normed, ctx, binding, into=ResidualTarget(residual, self.feed_forward_norm.lazy_params()))

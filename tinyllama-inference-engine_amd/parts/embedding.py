@@ -25,11 +25,13 @@ class TokenEmbedding(Part):
         self.table = None
 
     @classmethod
-    def tensor_specs(cls, spec, prefix=""):
-        return [TensorSpec(cls.NAME, (int(spec["vocab_size"]), int(spec["hidden_size"])))]
+    def tensor_specs(cls, spec, name=""):
+        """`name`: the table's full name in the checkpoint (the model's spec gives it; without one,
+        the reference's)."""
+        return [TensorSpec(name or cls.NAME, (int(spec["vocab_size"]), int(spec["hidden_size"])))]
 
-    def load(self, weights, prefix=""):
-        self.table = weights[self.NAME].contiguous()
+    def load(self, weights, name=""):
+        self.table = weights[name or self.NAME].contiguous()
 
     def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
         """The float32 residual [T, H] of the step's tokens.  `ctx` is the step's context: an
@@ -47,18 +49,21 @@ class LMHead(Part):
     NAME = "lm_head.weight"
 
     def __init__(self, spec: PartSpec, dtype, device):
+        """spec: vocab_size, hidden_size, tied (the head's matrix is the embedding's table), and, when
+        tied, optionally tied_to: that table's full name (default: the reference's)."""
         super().__init__(spec, dtype, device)
         self.tied = bool(spec.get("tied", False))
+        self.tied_to = spec.get("tied_to") or TokenEmbedding.NAME
         self.linear = None
 
     @classmethod
-    def tensor_specs(cls, spec, prefix=""):
+    def tensor_specs(cls, spec, name=""):
         shape = (int(spec["vocab_size"]), int(spec["hidden_size"]))
         # a tied model may still carry the head's matrix; it is then not read
-        return [TensorSpec(cls.NAME, shape, optional=bool(spec.get("tied", False)))]
+        return [TensorSpec(name or cls.NAME, shape, optional=bool(spec.get("tied", False)))]
 
-    def load(self, weights, prefix=""):
-        matrix = weights[TokenEmbedding.NAME] if self.tied else weights[self.NAME]
+    def load(self, weights, name=""):
+        matrix = weights[self.tied_to] if self.tied else weights[name or self.NAME]
         self.linear = Linear(matrix, None, self.dtype)
 
     def takes_normed_rows(self, rows: int) -> bool:

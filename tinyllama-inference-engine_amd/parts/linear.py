@@ -10,7 +10,7 @@ Which kernel runs is decided here and nowhere else:
   bfloat16, more rows            the library's product (as the reference uses a library for its
                                  products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out, or
                                  float32 for the output head: hipBLASLt called directly
-                                 (`ops.library_mm`), torch.mm where that fails
+                                 (`ops.library_mm`), the plain kernel where that fails
   anything those refuse          the plain kernel
 """
 from __future__ import annotations
@@ -65,12 +65,9 @@ class Linear:
             ops._device_tensor(x, "x", torch.bfloat16)
             if x.dim() != 2 or x.shape[1] != self.in_features:
                 raise ops.invalid_shape(f"linear: x {list(x.shape)} does not fit weight {list(self.weight.shape)}")
-            if out_dtype == torch.float32:              # (the output head's logits for many rows)
-                out = ops.library_mm(x, self.weight, torch.float32)
-                return Product(out + self.bias.float() if self.bias is not None else out, 1)
             if self.bias is not None:
-                # (the bias joins the float32 sums, as in the other kernels; element-wise kernels only, which a
-                # recording can hold: a library product with a bias has not been tried inside one)
-                return Product((ops.library_mm(x, self.weight, torch.float32) + self.bias.float()).to(torch.bfloat16), 1)
-            return Product(ops.library_mm(x, self.weight), 1)
+                # the library's product comes without the bias: it joins the float32 sums in a kernel of this
+                # library's own, as in the kernels that add it themselves, and the sum is rounded once
+                return Product(ops.add_bias(ops.library_mm(x, self.weight, torch.float32), self.bias, out_dtype), 1)
+            return Product(ops.library_mm(x, self.weight, out_dtype), 1)   # (float32: the output head's logits for many rows)
         return ops.gemm_generic(x, self.weight, self.bias, out_dtype)
