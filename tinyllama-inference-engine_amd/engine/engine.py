@@ -110,12 +110,14 @@ class Engine:
     def generate(self, prompts: Sequence[Sequence[int]], max_tokens: int = 16, temperature: float = 0.0,
                  top_p: float = 1.0, seed: int = 0, stop_on_eos: bool = False, max_tokens_per_step: int = 2048,
                  max_seqs_per_step: int | None = None, chunk_size: int | None = None,
-                 timings: dict | None = None) -> list[list[int]]:
+                 timings: dict | None = None, stats: dict | None = None) -> list[list[int]]:
         """Token ids in, generated token ids out, one list per prompt.  Request i samples with
         seed + i.  All prompts run together under the scheduler (continuous batching, prompts cut
         into portions under the token budget).  `timings`: a dict that receives the sums of the
         steps' compute and transfer times, apart for steps that bring prompt tokens and steps that
-        only decode (the keys of the reference's `generate`, app/cuda_reference.cu:216-224)."""
+        only decode (the keys of the reference's `generate`, app/cuda_reference.cu:216-224).
+        `stats`: a dict that receives what the scheduler counted (steps, prompt and decoded tokens,
+        preemptions)."""
         scheduler = Scheduler(self.cache, max_tokens_per_step=max_tokens_per_step,
                               max_seqs_per_step=max_seqs_per_step or self.cache.max_requests, chunk_size=chunk_size,
                               max_positions=self.spec.max_positions, eos_token_id=self.spec.eos_token_id)
@@ -128,6 +130,8 @@ class Engine:
             requests.append(request)
         try:
             self.run(scheduler, timings)
+            if stats is not None:
+                stats.update(scheduler.stats)
         except BaseException:
             # a step raised (no request can move, a NaN in the logits, a device error): what this
             # call's requests hold goes back, so that the engine can be used again
