@@ -218,3 +218,41 @@ def plain_generate_greedy(cfg: dict, w: dict, prompt: list[int], max_tokens: int
         generated.append(token)
         sequence.append(token)
     return generated
+
+
+def plain_forward_rows(cfg: dict, w: dict, tokens: list[int], rows: list[int]) -> torch.Tensor:
+    """Logits [len(rows), V] of a ONE-layer model at the chosen positions only: what `plain_forward`
+    gives at those rows, for sequences too long to compute whole.  Keys and values are made for
+    every position (they need only the embedding and the first norm), queries, attention, the
+    feed-forward and the head at the chosen rows; the same formulas as above, at the same places
+    of the reference (src/model.cpp:132-225)."""
+    assert cfg["num_hidden_layers"] == 1
+    heads = cfg["num_attention_heads"]
+    kv_heads = cfg.get("num_key_value_heads", heads)
+    head_dim = cfg.get("head_dim", cfg["hidden_size"] // heads)
+    eps, theta = cfg["rms_norm_eps"], cfg.get("rope_theta", 10000.0)
+    prefix = "model.layers.0."
+    count = len(tokens)
+    positions = torch.arange(count)
+    picked = torch.tensor(rows, dtype=torch.long)
+    x = w["model.embed_tokens.weight"].double()[torch.tensor(tokens, dtype=torch.long)]
+    normed = plain_rms_norm(x, w[prefix + "input_layernorm.weight"], eps)
+    k = plain_linear(normed, w[prefix + "self_attn.k_proj.weight"], w.get(prefix + "self_attn.k_proj.bias"))
+    v = plain_linear(normed, w[prefix + "self_attn.v_proj.weight"], w.get(prefix + "self_attn.v_proj.bias")).view(count, kv_heads, head_dim)
+    k = plain_rope(k.view(count, kv_heads, head_dim), positions, theta)
+    q = plain_linear(normed[picked], w[prefix + "self_attn.q_proj.weight"], w.get(prefix + "self_attn.q_proj.bias"))
+    q = plain_rope(q.view(len(rows), heads, head_dim), positions[picked], theta)
+    groups = heads // kv_heads
+    scale = 1.0 / math.sqrt(float(head_dim))
+    attended = torch.zeros(len(rows), heads, head_dim, dtype=torch.float64)
+    for index, t in enumerate(rows):
+        for head in range(heads):
+            scores = (k[:t + 1, head // groups] @ q[index, head]) * scale          # src/operators.cpp:119,131
+            attended[index, head] = plain_softmax(scores) @ v[:t + 1, head // groups]
+    x = x[picked] + plain_linear(attended.reshape(len(rows), heads * head_dim), w[prefix + "self_attn.o_proj.weight"],
+                                 w.get(prefix + "self_attn.o_proj.bias"))
+    normed = plain_rms_norm(x, w[prefix + "post_attention_layernorm.weight"], eps)
+    x = x + plain_linear(plain_silu_mul(plain_linear(normed, w[prefix + "mlp.gate_proj.weight"]),
+                                        plain_linear(normed, w[prefix + "mlp.up_proj.weight"])), w[prefix + "mlp.down_proj.weight"])
+    head_matrix = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
+    return plain_linear(plain_rms_norm(x, w["model.norm.weight"], eps), head_matrix)

@@ -90,8 +90,8 @@ def test_named_intermediate_tensors_layer_by_layer(setups, name, dtype):
     from tlie_amd import StepEntry
     engine.admit("t")
     first, second = {}, {}
-    engine.step([StepEntry("t", tokens[:30], list(range(30)))], trace=first)
-    engine.step([StepEntry("t", tokens[30:], list(range(15)))], trace=second)
+    engine.step([StepEntry("t", tokens[:28], list(range(28)))], trace=first)
+    engine.step([StepEntry("t", tokens[28:], list(range(17)))], trace=second)     # (17: more than the route of few rows takes)
     engine.finish("t")
     assert sorted(first) == sorted(plain) == sorted(second)
     order = ["embedding"] + [f"layer{layer}.{part}" for layer in range(layers)
@@ -106,6 +106,47 @@ def test_named_intermediate_tensors_layer_by_layer(setups, name, dtype):
     again = engine.step([StepEntry("u", tokens, list(range(45)))]).cpu()
     engine.finish("u")
     assert_close(again, torch.cat([first["logits"], second["logits"]]).cpu().double(), CUT_TOLERANCE[dtype], "without a trace")
+
+
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_named_intermediate_tensors_on_the_route_of_few_rows(setups, name):
+    """A bfloat16 step of at most 16 tokens (what decoding runs) folds the norms into its products
+    and lets the products add into the residual themselves; with a trace it takes that same route
+    and leaves what still exists there as a tensor: per layer what the mixer and the feed-forward
+    added and the layer's output, the embedding and the logits.  Steps of 9, 5, 1 and 1 tokens after
+    a prompt portion, each name against the plain implementation's rows at those positions."""
+    setup = setups(name, "bfloat16")
+    engine = new_engine(setup, "bfloat16")
+    tokens = request_tokens(name, 4, 45)
+    plain = {}
+    plain_forward(setup["raw"], setup["weights"], tokens, trace=plain)
+    layers = CONFIGS[name]["num_hidden_layers"]
+    from tlie_amd import StepEntry
+    engine.admit("t")
+    engine.step([StepEntry("t", tokens[:29], [])])
+    start, traces = 29, []
+    for count in (9, 5, 1, 1):
+        traces.append({})
+        engine.step([StepEntry("t", tokens[start:start + count], list(range(count)))], trace=traces[-1])
+        start += count
+    engine.finish("t")
+    names = ["embedding"] + [f"layer{layer}.{part}" for layer in range(layers) for part in ("attention_output", "mlp_output", "output")] \
+        + ["logits"]
+    for trace in traces:
+        assert sorted(trace) == sorted(names)          # the normed inputs do not exist on this route
+    for key in names:
+        got = torch.cat([trace[key] for trace in traces]).cpu()
+        assert got.dtype == torch.float32 and got.shape == plain[key][29:].shape, key
+        assert_close(got, plain[key][29:], TOLERANCE["bfloat16"], key)
+    # the same steps without a trace (replayed from recordings): the same logits up to the cut's tolerance
+    engine.admit("u")
+    engine.step([StepEntry("u", tokens[:29], [])])
+    again, start = [], 29
+    for count in (9, 5, 1, 1):
+        again.append(engine.step([StepEntry("u", tokens[start:start + count], list(range(count)))]).cpu())
+        start += count
+    engine.finish("u")
+    assert_close(torch.cat(again), torch.cat([trace["logits"] for trace in traces]).cpu().double(), CUT_TOLERANCE["bfloat16"], "without a trace")
 
 
 @pytest.mark.parametrize("name,dtype", CASES)

@@ -233,3 +233,23 @@ def test_model_trace_names_and_the_residual_sums():
         assert torch.allclose(trace[p + "input_norm"], plain_rms_norm(before, w[f"model.layers.{layer}.input_layernorm.weight"], 1e-5))
         before = trace[p + "output"]
     assert torch.allclose(trace["final_norm"], plain_rms_norm(before, w["model.norm.weight"], 1e-5))
+
+
+def test_rows_of_a_one_layer_model_are_the_whole_forward_at_those_rows():
+    """`plain_forward_rows` (for sequences too long to compute whole) against `plain_forward`."""
+    from plain_llama import plain_forward, plain_forward_rows
+    torch.manual_seed(3)
+    cfg = dict(hidden_size=48, intermediate_size=80, num_hidden_layers=1, num_attention_heads=6, num_key_value_heads=2, head_dim=8,
+               vocab_size=40, rms_norm_eps=1e-5, rope_theta=777.0, tie_word_embeddings=False)
+    p = "model.layers.0."
+    shapes = {"model.embed_tokens.weight": (40, 48), "lm_head.weight": (40, 48), "model.norm.weight": (48,),
+              p + "input_layernorm.weight": (48,), p + "post_attention_layernorm.weight": (48,),
+              p + "self_attn.q_proj.weight": (48, 48), p + "self_attn.k_proj.weight": (16, 48), p + "self_attn.v_proj.weight": (16, 48),
+              p + "self_attn.o_proj.weight": (48, 48), p + "self_attn.q_proj.bias": (48,), p + "self_attn.k_proj.bias": (16,),
+              p + "self_attn.v_proj.bias": (16,), p + "self_attn.o_proj.bias": (48,),
+              p + "mlp.gate_proj.weight": (80, 48), p + "mlp.up_proj.weight": (80, 48), p + "mlp.down_proj.weight": (48, 80)}
+    w = {name: torch.randn(shape, dtype=torch.float64) * 0.3 for name, shape in shapes.items()}
+    tokens = [(7 * i * i + 3) % 40 for i in range(33)]
+    whole = plain_forward(cfg, w, tokens)
+    rows = [0, 1, 16, 31, 32]
+    assert torch.allclose(plain_forward_rows(cfg, w, tokens, rows), whole[rows], rtol=1e-12, atol=1e-12)

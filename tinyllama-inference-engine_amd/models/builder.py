@@ -65,10 +65,11 @@ class DecoderModel:
         dict) the named tensors of the reference's ModelTrace are left there as float32 copies:
         "embedding", per run i "layer{i}.input_norm", ".attention_output", ".post_attention_norm",
         ".mlp_output", ".output", then "final_norm" and "logits" at the wanted rows
-        (src/model.cpp:98-231)."""
+        (src/model.cpp:98-231); a bfloat16 step of at most 16 tokens, which folds the norms into its
+        products, leaves the names that still exist as tensors on that route."""
         runs = self.spec.runs
         trace = getattr(ctx, "trace", None)
-        few = ops.few_rows_route(ctx.num_tokens, self.dtype) and trace is None
+        few = ops.few_rows_route(ctx.num_tokens, self.dtype)    # (also with a trace: it then shows the route that decoding takes)
 
         def entry_norm(block):
             # a block may say which norm reads the residual first (its writer can then leave that
@@ -97,7 +98,9 @@ class DecoderModel:
             normed = self.final_norm.add_forward(residual, pending, rows=ctx.want_rows)
         logits = self.head.forward(normed)
         if trace is not None:
-            trace["final_norm"], trace["logits"] = normed.float().clone(), logits.clone()
+            if isinstance(normed, torch.Tensor):             # (folded into the head's product on the route of few rows)
+                trace["final_norm"] = normed.float().clone()
+            trace["logits"] = logits.clone()
         return logits
 
 

@@ -62,23 +62,40 @@ class PreNormBlock:
         `next_norm`: the norm that reads the residual after this block, if the caller knows it.
         In a step of few rows the parts that offer it fold the norms into their products and add
         their results into the residual themselves; otherwise the norm kernels do both.
-        A step that keeps a trace (`ctx.trace`, a dict) takes the second way and leaves there, under
-        `ctx.trace_prefix`, the five tensors the reference's ModelTrace keeps per layer
-        (src/model.cpp:136-138,176-177,184-185,200-201,204-205), as float32 copies."""
-        if getattr(ctx, "trace", None) is not None:
-            return self._forward_traced(residual, pending, ctx, binding)
+        A step that keeps a trace (`ctx.trace`, a dict) leaves there, under `ctx.trace_prefix`, the
+        five tensors the reference's ModelTrace keeps per layer
+        (src/model.cpp:136-138,176-177,184-185,200-201,204-205), as float32 copies; on the route of
+        few rows, which it takes as a step without a trace would, those that still exist there:
+        "attention_output" and "mlp_output" (what the part added into the residual: the residual
+        after it minus the residual before) and "output" (the normed inputs are folded away)."""
+        trace = getattr(ctx, "trace", None)
         rows = residual.shape[0]
         few = ops.few_rows_route(rows, self.dtype)
+        if trace is not None and not few:
+            return self._forward_traced(residual, pending, ctx, binding)
+
+        def keep(name, tensor):
+            trace[ctx.trace_prefix + name] = tensor.float().clone()
         normed = self.mixer_norm.add_forward(residual, pending, lazy=few and self.mixer.takes_normed_rows(rows))
+        before = residual.clone() if trace is not None else None
         if few and self.mixer.adds_to_residual:
             mixed = self.mixer.forward(normed, ctx, binding, into=ResidualTarget(residual, self.feed_forward_norm.lazy_params()))
         else:
             mixed = self.mixer.forward(normed, ctx, binding)
         normed = self.feed_forward_norm.add_forward(residual, mixed, lazy=few and self.feed_forward.takes_normed_rows(rows))
+        if trace is not None:
+            keep("attention_output", residual - before)        # (whoever added it, the residual holds it now)
+            before = residual.clone()
         if few and self.feed_forward.adds_to_residual:
-            return self.feed_forward.forward(normed, ctx, into=ResidualTarget(
+            out = self.feed_forward.forward(normed, ctx, into=ResidualTarget(
                 residual, next_norm.lazy_params() if next_norm is not None else None))
-        return self.feed_forward.forward(normed, ctx)
+        else:
+            out = self.feed_forward.forward(normed, ctx)
+        if trace is not None:
+            added = residual - before if isinstance(out, ResidualUpdated) else as_product(out).dense(torch.float32)
+            keep("mlp_output", added)
+            keep("output", before + added)
+        return out
 
     def _forward_traced(self, residual, pending, ctx, binding):
         def keep(name, tensor):
