@@ -25,14 +25,14 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 HBM_PEAK = 8.0e12
 MFMA_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-# configs[2] of BASELINE.json: TinyLlama 1.1B
+# the TinyLlama 1.1B configuration
 TINYLLAMA = dict(model_type="llama", architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=5632,
                  num_hidden_layers=22, num_attention_heads=32, num_key_value_heads=4, max_position_embeddings=2048,
                  vocab_size=32000, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False, attention_bias=False,
                  hidden_act="silu", bos_token_id=1, eos_token_id=2, torch_dtype="bfloat16")
 
 
-# the layer sizes of BASELINE.json's configs[3] and configs[4], for `--shape`
+# the layer sizes of the Llama-2-7B and Llama-3-8B configurations, for `--shape`
 OTHER_SHAPES = {
     "llama2_7b": ("Llama-2-7B shape", dict(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
                                            num_key_value_heads=32, max_position_embeddings=4096, vocab_size=32000, rope_theta=10000.0)),

@@ -217,3 +217,15 @@ def test_random_orders_lose_nothing(seed):
         cache.release(request)
     cache.check()
     assert cache.free_pages() == [12] and cache.free_slots == 4
+
+
+def test_a_byte_budget_refuses_a_pool_before_it_is_allocated():
+    """src/kv_cache.cpp:40-43: more than the configured bytes is out_of_memory."""
+    needs = [RunNeed(0, KVCacheNeed(2, 8)), RunNeed(1, KVCacheNeed(2, 8)), RunNeed(0, KVCacheNeed(2, 8))]   # two pools, one reader
+    per_page = CacheManager.page_bytes(needs, 4, torch.float32)
+    assert per_page == 2 * (2 * 2 * 4 * 8 * 4)
+    CacheManager(needs, 4, 10, 2, torch.float32, "cpu", max_bytes=10 * per_page)
+    with pytest.raises(EngineError) as caught:
+        CacheManager(needs, 4, 11, 2, torch.float32, "cpu", max_bytes=10 * per_page)
+    assert caught.value.code == ErrorCode.OUT_OF_MEMORY and "budget" in caught.value.message
+    assert CacheManager.page_bytes(needs, 4, torch.bfloat16) == per_page // 2

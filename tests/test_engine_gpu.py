@@ -1010,3 +1010,23 @@ def test_several_prompts_from_the_command_line_batched_in_portions_with_preempti
     run = subprocess.run(cli + ["batch", setup["folder"], "20", "6", "0", "1", "--dtype", "float32", "--min-ratio", "1000"],
                          capture_output=True, text=True, timeout=300)
     assert run.returncode == 1 and json.loads(run.stdout)["passed"] is False
+
+
+def test_pool_sized_by_a_share_of_free_memory_and_byte_budgets(setups):
+    """Without a count of positions the pools take a share of the device memory that is free after
+    the weights; budgets in bytes refuse a folder or a pool with out_of_memory before anything is
+    mapped or allocated (src/weight_store.cpp:134-138, src/kv_cache.cpp:40-43)."""
+    from tlie_amd import Engine, EngineError, ErrorCode
+    setup = setups("A", "bfloat16")
+    free, _ = torch.cuda.mem_get_info()
+    engine = Engine(setup["folder"], dtype="bfloat16", max_tokens=None, cache_fraction=1e-4, max_requests=2)
+    per_page = engine.cache.page_bytes(engine.model.run_needs(), 16, torch.bfloat16)
+    assert per_page == 2 * (2 * 2 * 16 * 16 * 2)                       # two layers: keys and values of 2 heads of 16, 16 rows
+    assert 0.5e-4 * free / per_page < engine.cache.num_pages <= 1e-4 * free / per_page
+    assert engine.generate([[1, 2, 3]], max_tokens=4)[0] == new_engine(setup, "bfloat16").generate([[1, 2, 3]], max_tokens=4)[0]
+    for arguments in (dict(max_tokens=4096, max_cache_bytes=255 * per_page), dict(max_tokens=64, max_weight_file_bytes=1000)):
+        with pytest.raises(EngineError) as caught:
+            Engine(setup["folder"], dtype="bfloat16", **arguments)
+        assert caught.value.code == ErrorCode.OUT_OF_MEMORY and "budget" in caught.value.message
+    with pytest.raises(EngineError):
+        Engine(setup["folder"], dtype="bfloat16", max_tokens=None)

@@ -96,6 +96,36 @@ def test_tied_model_may_carry_its_head(tmp_path):
     tensors["lm_head.weight"] = torch.zeros(40, 32).bfloat16()
     write_safetensors(str(tmp_path / "model.safetensors"), tensors)
     WeightStore(str(tmp_path)).validate(specs)
+    # it is checked and not uploaded: the head reads the embedding's table
+    loaded = WeightStore(str(tmp_path)).load(specs, torch.bfloat16, "cpu")
+    assert "lm_head.weight" not in loaded and "model.embed_tokens.weight" in loaded
+    tensors["lm_head.weight"] = torch.zeros(41, 32).bfloat16()
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    assert code_of(lambda: WeightStore(str(tmp_path)).validate(specs)).code == ErrorCode.INVALID_SHAPE
+
+
+def test_matrices_stored_in_32_bit_stay_so_and_say_so(tmp_path):
+    """A tensor stored in 32-bit is kept in 32-bit also when the model runs in bfloat16 (its products
+    then take the true 32-bit kernel); the loader says so once, since nothing else would show it."""
+    import warnings
+    config = LlamaConfig.from_dict(TINY)
+    specs = expected_tensors(config.to_spec())
+    tensors = random_tensors(specs, seed=2)
+    name = "model.layers.0.mlp.down_proj.weight"
+    tensors[name] = tensors[name].float()
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()          # a vector: kept wide without a word
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        loaded = WeightStore(str(tmp_path)).load(specs, torch.bfloat16, "cpu")
+    assert loaded[name].dtype == torch.float32 and loaded["model.norm.weight"].dtype == torch.float32
+    assert loaded["model.layers.0.mlp.up_proj.weight"].dtype == torch.bfloat16
+    said = [str(warning.message) for warning in caught if "stored in 32-bit" in str(warning.message)]
+    assert len(said) == 1 and "1 matrices" in said[0] and name in said[0], [str(warning.message) for warning in caught]
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        WeightStore(str(tmp_path)).load(specs, torch.float32, "cpu")
+    assert not [warning for warning in caught if "stored in 32-bit" in str(warning.message)]
 
 
 def test_broken_files(tmp_path):
@@ -157,3 +187,15 @@ def test_checksum_of_the_weight_file(tmp_path):
     with pytest.raises(EngineError) as caught:
         store.expect_sha256("0" * 64)
     assert caught.value.code.value == "checksum_mismatch"
+
+
+def test_a_byte_budget_refuses_the_weight_files_before_mapping(tmp_path):
+    """src/weight_store.cpp:134-138: a file beyond the configured budget is out_of_memory."""
+    import os
+    config = LlamaConfig.from_dict(TINY)
+    specs = expected_tensors(config.to_spec())
+    write_safetensors(str(tmp_path / "model.safetensors"), random_tensors(specs, seed=3))
+    size = os.path.getsize(tmp_path / "model.safetensors")
+    WeightStore(str(tmp_path), max_file_bytes=size).validate(specs)
+    error = code_of(lambda: WeightStore(str(tmp_path), max_file_bytes=size - 1))
+    assert error.code == ErrorCode.OUT_OF_MEMORY and "budget" in error.message

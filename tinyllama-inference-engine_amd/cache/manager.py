@@ -56,12 +56,26 @@ class RequestPages:
 
 
 class CacheManager:
+    @staticmethod
+    def page_bytes(needs: list[RunNeed], page_size: int, dtype: torch.dtype) -> int:
+        """Bytes that one more page costs over all runs that own a pool (keys and values)."""
+        itemsize = torch.empty((), dtype=dtype).element_size()
+        return sum(2 * need.kv.num_kv_heads * page_size * need.kv.head_dim * itemsize
+                   for run, need in enumerate(needs) if need.kv is not None and need.cache_of == run)
+
     def __init__(self, needs: list[RunNeed], page_size: int, num_pages: int, max_requests: int,
-                 dtype: torch.dtype, device, max_positions: int | None = None):
+                 dtype: torch.dtype, device, max_positions: int | None = None, max_bytes: int | None = None):
+        """max_bytes: a budget for the pools; more is refused with `out_of_memory` before anything
+        is allocated (src/kv_cache.cpp:40-43)."""
         if page_size <= 0 or page_size & (page_size - 1):
             raise invalid_argument("page_size must be a power of two")
         if max_requests <= 0:
             raise invalid_argument("max_requests must be positive")
+        if num_pages <= 0:
+            raise invalid_argument("the cache needs at least one page")
+        if max_bytes is not None and num_pages * self.page_bytes(needs, page_size, dtype) > max_bytes:
+            raise out_of_memory(f"cache pools of {num_pages} pages take {num_pages * self.page_bytes(needs, page_size, dtype)} bytes, "
+                                f"which exceeds the configured budget of {max_bytes}")
         self.page_size = page_size
         self.num_pages = num_pages
         self.max_requests = max_requests

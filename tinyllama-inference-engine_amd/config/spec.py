@@ -91,4 +91,4 @@ class TensorSpec:
     name: str
     shape: tuple[int, ...]
     init: str = "normal"        # how random weights draw it: "normal", "norm" (around 1), "zeros"
-    optional: bool = False       # absent is not an error (a tied head that some files still carry)
+    optional: bool = False       # absent is no error, present it is checked and not read (a tied head's matrix that some files still carry)

@@ -37,12 +37,16 @@ def parse_dtype(name) -> torch.dtype:
 
 
 class Engine:
-    def __init__(self, model_dir: str | None, dtype="bfloat16", max_tokens: int = 4096, page_size: int = 16,
+    def __init__(self, model_dir: str | None, dtype="bfloat16", max_tokens: int | None = 4096, page_size: int = 16,
                  max_requests: int = 64, device: str = "cuda:0", config: dict | None = None,
                  random_seed: int | None = None, use_graphs: bool = True, expect_sha256: str | None = None,
-                 capture_graphs: bool = True):
+                 capture_graphs: bool = True, max_weight_file_bytes: int | None = None, max_cache_bytes: int | None = None,
+                 cache_fraction: float | None = None):
         """max_tokens: how many positions the cache pools hold in all (rounded up to whole
-        pages); max_requests: how many requests can be live at once.
+        pages); max_requests: how many requests can be live at once.  Instead of max_tokens
+        (None), cache_fraction sizes the pools as that share of the device memory that is free once
+        the weights are loaded.  max_weight_file_bytes and max_cache_bytes are budgets: a folder or
+        a pool beyond them is `out_of_memory` before anything is mapped or allocated.
 
         Without a folder, `config` (the contents of a config.json) and `random_seed` give a model
         of random weights drawn on the device, with no file in between (for measurements).
@@ -57,7 +61,7 @@ class Engine:
         if model_dir is not None:
             self.config = config_from_dict(read_config_json(model_dir))
             self.spec = self.config.to_spec()
-            store = WeightStore(model_dir)
+            store = WeightStore(model_dir, max_file_bytes=max_weight_file_bytes)
             if expect_sha256 is not None:
                 store.expect_sha256(expect_sha256)
             with device_memory_errors("the weights"):
@@ -72,12 +76,22 @@ class Engine:
                 weights = random_tensors(expected_tensors(self.spec), random_seed, dtype=self.dtype, device=self.device)
         with device_memory_errors("the weights"):
             self.model = build_model(self.spec, weights, self.dtype, self.device)
-        if max_tokens <= 0:
-            raise invalid_argument("max_tokens must be positive")
-        num_pages = (max_tokens + page_size - 1) // page_size
+        needs = self.model.run_needs()
+        if max_tokens is None:
+            if cache_fraction is None or not 0.0 < cache_fraction <= 1.0:
+                raise invalid_argument("without max_tokens the engine needs a cache_fraction in (0, 1]")
+            free, _ = torch.cuda.mem_get_info(self.device)
+            per_page = CacheManager.page_bytes(needs, page_size, self.dtype)
+            num_pages = int(free * cache_fraction) // per_page if per_page else 1
+            if num_pages <= 0:
+                raise EngineError(ErrorCode.OUT_OF_MEMORY, f"{cache_fraction} of the {free} free bytes do not hold one page of {per_page}")
+        else:
+            if max_tokens <= 0:
+                raise invalid_argument("max_tokens must be positive")
+            num_pages = (max_tokens + page_size - 1) // page_size
         with device_memory_errors(f"cache pools of {num_pages} pages"):
-            self.cache = CacheManager(self.model.run_needs(), page_size, num_pages, max_requests, self.dtype, self.device,
-                                      max_positions=self.spec.max_positions)
+            self.cache = CacheManager(needs, page_size, num_pages, max_requests, self.dtype, self.device,
+                                      max_positions=self.spec.max_positions, max_bytes=max_cache_bytes)
         self.runner = ModelRunner(self.model, self.cache, use_graphs=use_graphs, capture=capture_graphs)
         self.sampler = Sampler(self.device, capacity=max(max_requests, 1))
         self.runner.device_tokens = self.sampler.device_tokens

@@ -29,7 +29,9 @@ _IGNORED = (re.compile(r".*\.rotary_emb\.inv_freq$"),)
 class WeightStore:
     """All safetensors files of a model folder behind one `get(name)`."""
 
-    def __init__(self, model_dir: str):
+    def __init__(self, model_dir: str, max_file_bytes: int | None = None):
+        """max_file_bytes: a budget for the weight files together; a folder beyond it is refused
+        with `out_of_memory` before any file is mapped (src/weight_store.cpp:134-138)."""
         self.model_dir = model_dir
         self._files: list[SafetensorsFile] = []
         self._where: dict[str, SafetensorsFile] = {}
@@ -46,6 +48,14 @@ class WeightStore:
             names = ["model.safetensors"]
         else:
             raise EngineError(ErrorCode.IO, f"unable to open weights: {single} does not exist")
+        if max_file_bytes is not None:
+            try:
+                total = sum(os.path.getsize(os.path.join(model_dir, name)) for name in names)
+            except OSError as error:
+                raise EngineError(ErrorCode.IO, f"unable to stat the weight files of {model_dir} ({error.strerror})") from None
+            if total > max_file_bytes:
+                raise EngineError(ErrorCode.OUT_OF_MEMORY, f"the weight files hold {total} bytes, which exceeds the configured "
+                                                           f"budget of {max_file_bytes} before mapping")
         for name in names:
             file = SafetensorsFile(os.path.join(model_dir, name))
             self._files.append(file)
@@ -109,13 +119,25 @@ class WeightStore:
                               f"weights in {self.model_dir} do not fit the model — " + " | ".join(parts))
 
     def load(self, specs: Iterable[TensorSpec], dtype: torch.dtype, device) -> dict[str, torch.Tensor]:
-        """Validates, then uploads every expected tensor that is present, in its kept precision."""
+        """Validates, then uploads every required tensor, in its kept precision.  A tensor the
+        model marks optional (a tied head's matrix that some files still carry) is checked when
+        present and not uploaded: no part reads it.  A matrix stored in 32-bit stays 32-bit also in
+        a bfloat16 run (its products then go to the true 32-bit kernel, at a fraction of the
+        speed): that is said once, as a warning, because nothing else shows it."""
         specs = list(specs)
         self.validate(specs)
-        out = {}
+        out, wide = {}, []
         for spec in specs:
-            if spec.name in self._where:
-                out[spec.name] = to_kept_precision(self.get(spec.name), dtype).to(device)
+            if spec.name in self._where and not spec.optional:
+                kept = to_kept_precision(self.get(spec.name), dtype)
+                if dtype == torch.bfloat16 and kept.dtype == torch.float32 and kept.dim() >= 2:
+                    wide.append(spec.name)
+                out[spec.name] = kept.to(device)
+        if wide:
+            import warnings
+            warnings.warn(f"{len(wide)} matrices of {self.model_dir} are stored in 32-bit and are kept so in this bfloat16 run "
+                          f"(first: {wide[0]}); their products take the 32-bit kernel, which is many times slower",
+                          stacklevel=2)
         return out
 
 
