@@ -30,7 +30,9 @@
 //    before it knows how long the sequence is: the position, the block table and the keys are not
 //    three loads in a row.
 #include "common.h"
+#include "no_alloc.h"
 
+#include <mutex>
 #include <type_traits>
 
 namespace tlie {
@@ -651,10 +653,10 @@ using namespace tlie;
 // takes 16 * col_tiles of them, and keys and values reach the waves through LDS.  Otherwise:
 // waves: 1, 2, 4 or 8 waves of a workgroup share a tile's keys; waves * col_tiles * d <= 1024 (their merge's LDS), and
 // at most 4 when col_tiles * d > 128.
-extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
-                                   const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
-                                   float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
-                                   int d, int page_size, int window, float scale, int waves, int shared, void* stream) {
+static int attention_entry(const void* q, const void* cache, const int* block_table, int max_blocks,
+                           const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
+                           float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
+                           int d, int page_size, int window, float scale, int waves, int shared, void* stream) {
   if (num_tiles <= 0 || tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || d % 16 != 0 ||
       page_size < 16 || (page_size & (page_size - 1)) != 0 || max_blocks <= 0 || nsplit < 1 || nsplit > 65535 || nkv > 65535)
     return kBadArgument;
@@ -714,4 +716,56 @@ extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* 
   hipLaunchKernelGGL(attention_merge_kernel, dim3(tokens * nq), dim3(64), nsplit * sizeof(float), s, part_o, part_ml,
                      (uint16_t*)out, nsplit, d);
   return launch_status();
+}
+
+extern "C" int tlie_attention_mfma(const void* q, const void* cache, const int* block_table, int max_blocks,
+                                   const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
+                                   float* part_o, float* part_ml, int nsplit, int split_len, int tokens, int nq, int nkv,
+                                   int d, int page_size, int window, float scale, int waves, int shared, void* stream) {
+  return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
+                         split_len, tokens, nq, nkv, d, page_size, window, scale, waves, shared, stream);
+}
+
+// ---- the same attention for callers that cannot allocate (declared and described in no_alloc.h) ----------
+// The partial results of the key parts (what `part_o` and `part_ml` bring in above) live in this array, of
+// which every GPU the library runs on holds its own copy until the process ends.
+static __device__ __align__(256) unsigned char scratch[TLIE_NO_ALLOC_SCRATCH_BYTES];
+
+// In host code the array's name is only a stand-in for the symbol: its device address is asked for once
+// per device, with that device current, and kept; kernels are handed that address, never the name.
+static void* scratch_address() {
+  static std::mutex guard;
+  static void* address[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(guard);
+  if (address[device] == nullptr) {
+    void* found = nullptr;
+    if (hipGetSymbolAddress(&found, HIP_SYMBOL(scratch)) != hipSuccess || found == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    address[device] = found;
+  }
+  return address[device];
+}
+
+extern "C" int tlie_attention_mfma_no_alloc(const void* q, const void* cache, const int* block_table, int max_blocks,
+                                            const void* tiles, int num_tiles, int col_tiles, const int* positions, void* out,
+                                            int nsplit, int split_len, int tokens, int nq, int nkv, int d, int page_size,
+                                            int window, float scale, int waves, int shared, void* stream) {
+  if (tokens <= 0 || nq <= 0 || d <= 0 || nsplit < 1) return kBadArgument;
+  float *part_o = nullptr, *part_ml = nullptr;
+  if (nsplit > 1) {
+    // [tokens * nq * nsplit] rows of d floats, then as many pairs (maximum, sum), the pairs at a multiple of 256 bytes
+    const size_t rows = static_cast<size_t>(tokens) * nq * nsplit;
+    const size_t o_bytes = (rows * d * sizeof(float) + 255) / 256 * 256;
+    if (o_bytes + rows * 2 * sizeof(float) > TLIE_NO_ALLOC_SCRATCH_BYTES) return kScratchTooSmall;
+    unsigned char* base = static_cast<unsigned char*>(scratch_address());
+    if (base == nullptr) return kLaunchFailed;
+    part_o = reinterpret_cast<float*>(base);
+    part_ml = reinterpret_cast<float*>(base + o_bytes);
+  }
+  return attention_entry(q, cache, block_table, max_blocks, tiles, num_tiles, col_tiles, positions, out, part_o, part_ml, nsplit,
+                         split_len, tokens, nq, nkv, d, page_size, window, scale, waves, shared, stream);
 }

@@ -122,6 +122,7 @@ __device__ __forceinline__ float sum_splits(const D* __restrict__ first, int nsp
 constexpr int kOk = 0;
 constexpr int kBadArgument = -1;   // a size or dtype the kernel does not take
 constexpr int kLaunchFailed = -2;  // hipGetLastError() reported an error after the launch
+constexpr int kScratchTooSmall = -4;  // the sizes need more scratch memory than the library's own array holds
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? kOk : kLaunchFailed; }
 
