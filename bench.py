@@ -170,6 +170,10 @@ def main() -> int:
                              "continuously; mixed: 8 prompts of 8192 tokens in portions beside 56 short decode streams "
                              "(needs a shape with 8192 positions); each prints a record of its own")
     parser.add_argument("--token-budget", type=int, default=2048, help="tokens a step of a workload may hold")
+    parser.add_argument("--kernels", nargs="?", const="", default=None, metavar="NAME",
+                        help="time the kernels of a decode step (--batch, --context) and of a prompt step one by one at the "
+                             "shape's layer sizes, each inside a replayed recording that walks through copies of its weights; "
+                             "NAME keeps the kernels whose name holds it; prints one JSON line per kernel")
     parser.add_argument("--shape", default="tinyllama", choices=["tinyllama", *OTHER_SHAPES],
                         help="layer sizes of another model of the same architecture (the default is the record's)")
     args = parser.parse_args()
@@ -190,6 +194,11 @@ def main() -> int:
         return 2
     itemsize = 2 if args.dtype == "bfloat16" else 4
     vocab = cfg["vocab_size"]
+    if args.kernels is not None:
+        from tlie_amd.kernel_bench import bench_kernels
+        for row in bench_kernels(cfg, batch=args.batch, context=args.context, prompt=args.prefill or 2048, only=args.kernels or None):
+            print(json.dumps(row), flush=True)
+        return 0
     if args.workload != "decode":
         if args.workload == "mixed" and cfg["max_position_embeddings"] < 8192:
             print("the mixed workload has prompts of 8192 tokens: take --shape llama3_8b")

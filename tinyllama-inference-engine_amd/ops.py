@@ -774,3 +774,40 @@ def embed_rows(tokens: torch.Tensor, table: torch.Tensor, next_norm: tuple):
                                      dtype_code(next_weight.dtype), _ptr(xg), _ptr(ssq), count, hidden, _stream()),
            "embed_rows")
     return residual, NormedRows(xg, ssq, float(next_eps))
+
+
+# ---- the machine's own ceilings ---------------------------------------------------------------------
+def measured_peaks(device="cuda:0", repeats: int = 5) -> dict:
+    """What this GPU delivers to kernels that do nothing else: GB/s of a streaming read of 2 GiB
+    (workgroups of 512 threads, four a compute unit, eight 16-byte loads in flight a thread) and
+    TFLOP/s of chains of bfloat16 matrix instructions (32 x 32 x 16, eight independent chains a wave,
+    eight waves a compute unit); the best of `repeats` timed launches each, after one warm-up."""
+    device = torch.device(device)
+    units = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    sink = torch.zeros(4, dtype=torch.float32, device=device)
+    data = torch.empty(1 << 31, dtype=torch.uint8, device=device)
+    data.fill_(1)
+    blocks = 4 * units
+    lib = library()
+    lib.tlie_probe_stream_read_bytes.restype = ctypes.c_ulonglong
+    read_bytes = lib.tlie_probe_stream_read_bytes(ctypes.c_ulonglong(data.numel()), blocks)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best_read = best_mfma = None
+    iterations, mfma_blocks = 4096, 2 * units
+    for run in range(repeats + 1):
+        start.record()
+        _check(lib.tlie_probe_stream_read(_ptr(data), ctypes.c_ulonglong(data.numel()), blocks, _ptr(sink), _stream()), "probe_stream_read")
+        stop.record()
+        stop.synchronize()
+        seconds = start.elapsed_time(stop) / 1e3
+        if run > 0:
+            best_read = seconds if best_read is None else min(best_read, seconds)
+        start.record()
+        _check(lib.tlie_probe_mfma_bf16(iterations, mfma_blocks, _ptr(sink), _stream()), "probe_mfma_bf16")
+        stop.record()
+        stop.synchronize()
+        seconds = start.elapsed_time(stop) / 1e3
+        if run > 0:
+            best_mfma = seconds if best_mfma is None else min(best_mfma, seconds)
+    flops = mfma_blocks * 4 * 8 * iterations * 32768.0
+    return {"stream_read_gbs": read_bytes / best_read / 1e9, "mfma_bf16_tflops": flops / best_mfma / 1e12}
