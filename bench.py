@@ -8,11 +8,18 @@
 A step is one decode step of the whole batch.  The batch's requests are first prefilled so that
 after the warm-up and the K timed steps their length is `context`; then W untimed and exactly K
 timed steps run, each through the engine's own step function and sampler (greedy), and one JSON
-line is printed.  `value` is decoded tokens per second.  The same line carries the prefill of a
-2,048-token prompt, the decode step's share of the HBM roofline, and decoding at batch 1 and 64.
+line is printed; that is done `--repeats` times and the median run counts.  `value` is decoded
+tokens per second.  The same line carries the prefill of a 2,048-token prompt, the decode step's
+share of the HBM roofline, and in `points` (every key a number): decoding at batch 1 and 64, the
+workload of a 128-token prompt with 128 generated tokens, the same model in true 32-bit (decoding and
+the prompt step), and decoding at the layer sizes of Llama-2-7B and Llama-3-8B with a quarter of
+their layers (the counts are named); `*_frac` is the share of the published peak (HBM for decoding,
+the matrix cores of the dtype for prompts).
 
 Peaks are the MI355X's published ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bfloat16, 157.3
-TFLOP/s for float32.
+TFLOP/s for float32.  `measured_peaks` holds what two microbenchmarks of the kernel library reach
+on the machine at hand (a streaming read, chains of bfloat16 matrix instructions), and
+`frac_of_measured` the same shares against those.
 """
 import argparse
 import json
@@ -160,6 +167,8 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--context", type=int, default=2048)
+    parser.add_argument("--repeats", type=int, default=3,
+                        help="the timed steps are run so many times, each after prompts and warm-up of its own; the median is reported")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--layers", type=int, default=0, help="run fewer layers than the configuration has (named in the record)")
     parser.add_argument("--no-points", action="store_true", help="skip batch 1 and 64 and the prefill")
@@ -223,20 +232,29 @@ def main() -> int:
                           "frac": prefill_flops(cfg, args.prefill) / seconds / MFMA_PEAK[args.dtype]}))
         return 0
     most = max(args.batch, 1 if args.no_points else 64)
+    started_all = time.perf_counter()
     engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=most * args.context + 2048,
                     page_size=16, max_requests=most + 1)
 
-    elapsed = time_decode(engine, torch, args.batch, args.context, args.steps, args.warmup, vocab)
+    def median_decode(engine, batch, context, steps, warmup, vocab, repeats):
+        """Seconds for `steps` timed decode steps: the median of `repeats` runs, each with its own
+        prompts and `warmup` untimed steps before the timed ones."""
+        runs = sorted(time_decode(engine, torch, batch, context, steps, warmup, vocab) for _ in range(repeats))
+        return runs[len(runs) // 2]
+
+    def step_bytes(cfg, itemsize, batch, context, steps):
+        return weight_bytes_per_step(cfg, itemsize) + batch * (context - steps / 2) * kv_bytes_per_token(cfg, itemsize)
+
+    elapsed = median_decode(engine, args.batch, args.context, args.steps, args.warmup, vocab, args.repeats)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
-    mean_context = args.context - args.steps / 2
-    step_bytes = weight_bytes_per_step(cfg, itemsize) + args.batch * mean_context * kv_bytes_per_token(cfg, itemsize)
-    achieved = step_bytes / (elapsed / args.steps)
+    achieved = step_bytes(cfg, itemsize, args.batch, args.context, args.steps) / (elapsed / args.steps)
     record = {
         "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({model_name})", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "repeats": args.repeats,            # the timed steps were run so many times, each after its own warm-up; the median counts
         "config": {"model": model_name, "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
                    "hidden": cfg["hidden_size"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["hidden_size"] // cfg["num_attention_heads"], "ffn": cfg["intermediate_size"],
@@ -246,18 +264,67 @@ def main() -> int:
                      "frac": achieved / HBM_PEAK},
     }
     if not args.no_points:
+        from tlie_amd import ops
+        peaks = ops.measured_peaks(engine.device)
+        record["measured_peaks"] = {"stream_read_gbs": peaks["stream_read_gbs"], "mfma_bf16_tflops": peaks["mfma_bf16_tflops"]}
+        record["roofline"]["frac_of_measured"] = achieved / (peaks["stream_read_gbs"] * 1e9)
         prefill_tokens = 2048
         seconds = time_prefill(engine, torch, prefill_tokens, vocab)
+        flops = prefill_flops(cfg, prefill_tokens)
         record["prefill"] = {"value": prefill_tokens / seconds, "tokens": prefill_tokens, "ms": seconds * 1e3,
-                             "frac": prefill_flops(cfg, prefill_tokens) / seconds / MFMA_PEAK[args.dtype]}
+                             "frac": flops / seconds / MFMA_PEAK[args.dtype]}
+        if args.dtype == "bfloat16":
+            record["prefill"]["frac_of_measured"] = flops / seconds / (peaks["mfma_bf16_tflops"] * 1e12)
         points = {}
         for batch in (1, 64):
             steps = min(args.steps, 64)
-            seconds = time_decode(engine, torch, batch, args.context, steps, 4, vocab)
+            seconds = median_decode(engine, batch, args.context, steps, 4, vocab, args.repeats)
             points[f"decode_b{batch}"] = batch * steps / seconds
+            points[f"decode_b{batch}_frac"] = step_bytes(cfg, itemsize, batch, args.context, steps) / (seconds / steps) / HBM_PEAK
         # a short prompt: its step is replayed from a recording (the long one's is launched kernel by kernel)
         points["prefill_256"] = 256 / time_prefill(engine, torch, 256, vocab)
+        # the workload of a prompt of 128 tokens and 128 generated ones, at the record's batch
+        warm = 8
+        timed = 128 - warm - 1
+        seconds = median_decode(engine, args.batch, 256, timed, warm, vocab, args.repeats)
+        points[f"decode_b{args.batch}_prompt128"] = args.batch * timed / seconds
+        points[f"decode_b{args.batch}_prompt128_frac"] = step_bytes(cfg, itemsize, args.batch, 256, timed) / (seconds / timed) / HBM_PEAK
+        del engine
+        torch.cuda.empty_cache()
+        if args.dtype == "bfloat16" and args.shape == "tinyllama":
+            # the same model in true 32-bit (the check path): decoding at the record's batch and the prompt step
+            wide = Engine(None, dtype="float32", config=cfg, random_seed=0, max_tokens=args.batch * args.context + 4096,
+                          page_size=16, max_requests=args.batch + 1)
+            steps = 24
+            seconds = median_decode(wide, args.batch, args.context, steps, 2, vocab, args.repeats)
+            points[f"fp32_decode_b{args.batch}"] = args.batch * steps / seconds
+            points[f"fp32_decode_b{args.batch}_frac"] = step_bytes(cfg, 4, args.batch, args.context, steps) / (seconds / steps) / HBM_PEAK
+            seconds = time_prefill(wide, torch, prefill_tokens, vocab, repeats=2)
+            points["fp32_prefill_2048"] = prefill_tokens / seconds
+            points["fp32_prefill_2048_frac"] = flops / seconds / MFMA_PEAK["float32"]
+            del wide
+            torch.cuda.empty_cache()
+            # the layer sizes of the two larger models of the same architecture, a quarter of their layers
+            # (named beside the number), decoding at the record's batch at 2048 positions
+            for shape, (name, sizes) in OTHER_SHAPES.items():
+                larger = dict(TINYLLAMA)
+                larger.update(sizes)
+                layers_of_model = larger["num_hidden_layers"]
+                larger["num_hidden_layers"] = layers_of_model // 4
+                other = Engine(None, dtype="bfloat16", config=larger, random_seed=0, max_tokens=args.batch * 2048 + 2048,
+                               page_size=16, max_requests=args.batch + 1)
+                steps = 32
+                seconds = median_decode(other, args.batch, 2048, steps, 4, larger["vocab_size"], args.repeats)
+                key = f"{shape}_decode_b{args.batch}"
+                points[key] = args.batch * steps / seconds
+                points[key + "_ms"] = seconds / steps * 1e3
+                points[key + "_frac"] = step_bytes(larger, 2, args.batch, 2048, steps) / (seconds / steps) / HBM_PEAK
+                points[key + "_layers"] = larger["num_hidden_layers"]
+                points[key + "_layers_of_model"] = layers_of_model
+                del other
+                torch.cuda.empty_cache()
         record["points"] = points
+        record["bench_seconds"] = time.perf_counter() - started_all
     print(json.dumps(record))
     return 0
 
