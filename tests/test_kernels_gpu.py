@@ -228,6 +228,51 @@ def test_attention_generic(dtype, case):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", [
+    dict(nq=8, nkv=2, d=64, page=16, window=None), dict(nq=6, nkv=3, d=48, page=16, window=70),
+    dict(nq=5, nkv=5, d=7, page=8, window=None), dict(nq=40, nkv=1, d=16, page=16, window=300),   # 40 heads a group: two blocks of heads
+])
+def test_attention_that_shares_keys_among_neighbouring_tokens_gives_the_same_bits(dtype, case):
+    """The plain attention kernel has a form for steps whose sequences bring several tokens: a
+    workgroup serves up to 32 (token, head) columns and reads each chunk of keys once for all of
+    them.  A column's arithmetic is the same operation for operation, so the two forms must agree in
+    every bit, whatever the step: here portions of three sequences of different lengths (one of
+    them a single token, one starting mid-way), tokens of different sequences falling into one
+    workgroup; and both agree with the plain implementation."""
+    from tlie_amd import ops
+    nq, nkv, d, page, window = case["nq"], case["nkv"], case["d"], case["page"], case["window"]
+    torch.manual_seed(nq * 100 + d)
+    lengths, firsts = [613, 1, 290], [0, 0, 201]                  # the step brings positions firsts[i] .. lengths[i] - 1
+    padding = 5                                                   # tokens of the first sequence again, at position 0, at the step's end (a recording's padding)
+    caches, tables, offset = [], [], 0
+    qs, wants, token_seq, positions = [], [], [], []
+    for index, (length, first) in enumerate(zip(lengths, firsts)):
+        q, k, v = torch.randn(length, nq, d), torch.randn(length, nkv, d), torch.randn(length, nkv, d)
+        cache, pages = build_cache(k, v, page, DT[dtype], shuffle_seed=index)
+        caches.append(cache)
+        tables.append([page_index + offset for page_index in pages])
+        offset += cache.shape[0]
+        qs.append(q[first:])
+        wants.append(plain_attention(rounded(q, DT[dtype]), rounded(k, DT[dtype]), rounded(v, DT[dtype]), window=window)[first:])
+        token_seq += [index] * (length - first)
+        positions += list(range(first, length))
+    qs.append(torch.randn(padding, nq, d))
+    token_seq += [0] * padding
+    positions += [0] * padding
+    width = max(len(row) for row in tables)
+    table = torch.tensor([row + [0] * (width - len(row)) for row in tables], dtype=torch.int32, device=DEV)
+    cache = torch.cat(caches).to(DEV)
+    q = torch.cat(qs).to(DT[dtype]).reshape(-1, nq * d).to(DEV).contiguous()
+    arguments = (q, cache, table, torch.tensor(token_seq, dtype=torch.int32, device=DEV),
+                 torch.tensor(positions, dtype=torch.int32, device=DEV), nq, nkv, d, window, 1.0 / math.sqrt(d))
+    alone = ops.attention_generic(*arguments, tiled=False)
+    shared = ops.attention_generic(*arguments, tiled=True)
+    assert torch.isfinite(shared.float()).all()
+    assert torch.equal(alone, shared)
+    assert rel_err(shared.view(-1, nq, d)[:-padding], torch.cat(wants)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_attention_finds_one_key_among_hundreds(dtype):
     """One key is made to stand out (its score is far above the rest), at places where an index
     mistake would miss it: the first key, a page's last row and the next page's first, the last

@@ -117,6 +117,172 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
   }
 }
 
+// The same attention for steps that bring several tokens of a sequence (prompt portions): a
+// workgroup serves up to 32 columns, a column being a (token, query head) pair, of up to 32 / heads
+// consecutive tokens of the step and the heads of one kv head (or 32 of them), and brings every
+// chunk of 64 keys and values through LDS once for all of them, where the kernel above reads
+// each key and value again for every column (a prompt of 2048 tokens: 34 GB of cache traffic a layer).
+//
+// The arithmetic of a column is the kernel's above, operation for operation: chunk c of the context
+// belongs to running state c % 4 (there: to thread group c % 4), a chunk's scores are 64 dot products
+// summed in the order of the dims, its maximum and sum are the same reductions over a wave, the
+// values are added in the order of the keys, and the four states meet in the same order at the end.
+// A column therefore gets the same bits from either kernel, and a step may take whichever is faster.
+// Head sizes up to 64.  Tokens of a workgroup that belong to different sequences are served one
+// run of equal sequences after the other.
+constexpr int kTiledCols = 32, kTiledSlots = 8;     // columns a workgroup, columns a wave
+template <typename T>
+__global__ void __launch_bounds__(256)
+attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
+                               int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
+                               T* __restrict__ out, int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
+                               int tokens_per_block, int heads_per_block) {
+  extern __shared__ float lds[];
+  const int k_stride = d | 1;                      // odd: the 64 lanes of a wave read 64 different banks
+  float* k_tile = lds;                             // [64 keys][k_stride]
+  float* v_tile = k_tile + 64 * k_stride;          // [d][65]
+  float* q_tile = v_tile + d * 65;                 // [32 columns][d]
+  float* prob = q_tile + kTiledCols * d;           // [4 waves][4 columns][64 keys]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int G = nq / nkv, kv_head = blockIdx.y;
+  const int tok0 = blockIdx.x * tokens_per_block, head0 = blockIdx.z * heads_per_block;
+  const int ntok = min(tokens_per_block, tokens - tok0), nheads = min(heads_per_block, G - head0);
+  const int ncols = ntok * nheads;                 // column c = (token c / nheads, head c % nheads)
+  const size_t page_stride = static_cast<size_t>(2) * nkv * page_size * d;
+  const size_t head_offset = static_cast<size_t>(kv_head) * page_size * d;
+  const size_t v_offset = static_cast<size_t>(nkv) * page_size * d;
+
+  for (int e = threadIdx.x; e < ncols * d; e += 256) {
+    const int c = e / d, i = e - c * d;
+    q_tile[c * d + i] = to_float(q[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * d + i]);
+  }
+  // this wave's columns: slot s is column wave + 4 s
+  int col_pos[kTiledSlots], col_lo[kTiledSlots], col_tok[kTiledSlots];     // col_tok: the column's token among the workgroup's, or -1
+#pragma unroll
+  for (int s = 0; s < kTiledSlots; ++s) {
+    const int c = wave + 4 * s;
+    const bool live = c < ncols;
+    col_tok[s] = live ? c / nheads : -1;
+    col_pos[s] = live ? positions[tok0 + col_tok[s]] : -1;
+    col_lo[s] = live && window > 0 ? max(0, col_pos[s] - window + 1) : 0;
+  }
+  float run_max[4][kTiledSlots], run_sum[4][kTiledSlots], acc[4][kTiledSlots];
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int s = 0; s < kTiledSlots; ++s) run_max[g][s] = -INFINITY, run_sum[g][s] = 0.f, acc[g][s] = 0.f;
+
+  // runs of tokens of one sequence, in the order of the tokens (a column belongs to the run its token
+  // lies in: a sequence may come twice among a workgroup's tokens, when a recorded step pads its
+  // tokens with tokens of its first sequence)
+  int run_first = 0;
+  while (run_first < ntok) {                       // (the same for every thread: the barriers below are the workgroup's)
+    const int seq = token_seq[tok0 + run_first];
+    int run_end = run_first + 1;
+    while (run_end < ntok && token_seq[tok0 + run_end] == seq) ++run_end;
+    // the keys the run's columns see: from the least lower bound to the last token's position
+    int hi = -1, lo = 1 << 30;
+    for (int t = run_first; t < run_end; ++t) {
+      const int pos = positions[tok0 + t];
+      hi = max(hi, pos);
+      lo = min(lo, window > 0 ? max(0, pos - window + 1) : 0);
+    }
+    const int* pages = block_table + static_cast<size_t>(seq) * max_blocks;
+    for (int base = (lo / 256) * 256; base <= hi; base += 256) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int start = base + g * 64;
+        if (start > hi) break;                     // (uniform)
+        __syncthreads();                           // the tiles of the chunk before have been read
+        for (int e = threadIdx.x; e < 64 * d; e += 256) {
+          const int r = e / d, i = e - r * d, j = start + r;
+          if (j <= hi && j >= lo)
+            k_tile[r * k_stride + i] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + head_offset +
+                                                      static_cast<size_t>(j % page_size) * d + i]);
+        }
+        for (int e = threadIdx.x; e < 64 * d; e += 256) {
+          const int dim = e >> 6, r = e & 63, j = start + r;
+          if (j <= hi && j >= lo)
+            v_tile[dim * 65 + r] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + v_offset + head_offset +
+                                                  static_cast<size_t>(dim) * page_size + j % page_size]);
+        }
+        __syncthreads();
+        // four columns at a time: their dot products share each read of a key, and the chains of
+        // additions of one column wait for each other less
+#pragma unroll
+        for (int b = 0; b < kTiledSlots / 4; ++b) {
+          bool any = false;
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+            any |= col_tok[b * 4 + u] >= run_first && col_tok[b * 4 + u] < run_end && col_pos[b * 4 + u] >= start && col_lo[b * 4 + u] < start + 64;
+          if (!any) continue;                      // (uniform over the wave: the columns are the wave's)
+          const int j = start + lane;
+          float dot[4] = {0.f, 0.f, 0.f, 0.f};
+          const float* key = k_tile + lane * k_stride;
+          for (int i = 0; i < d; ++i) {
+            const float kv = key[i];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) dot[u] += q_tile[min(wave + 4 * (b * 4 + u), kTiledCols - 1) * d + i] * kv;
+          }
+          float* my_prob = prob + (wave * 4) * 64;
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int s = b * 4 + u;
+            const bool column = col_tok[s] >= run_first && col_tok[s] < run_end && col_pos[s] >= start && col_lo[s] < start + 64;   // a chunk without keys changes nothing
+            if (!column) continue;                 // (uniform over the wave)
+            const bool valid = j >= col_lo[s] && j <= col_pos[s];
+            const float score = valid ? dot[u] * scale : -INFINITY;
+            const float new_max = fmaxf(run_max[g][s], wave_max(score));
+            const float p = valid ? expf(score - new_max) : 0.f;
+            my_prob[u * 64 + lane] = p;
+            const float chunk_sum = wave_sum(p);
+            const float alpha = new_max == -INFINITY ? 1.f : expf(run_max[g][s] - new_max);
+            run_sum[g][s] = run_sum[g][s] * alpha + chunk_sum;
+            run_max[g][s] = new_max;
+            acc[g][s] *= alpha;
+          }
+          // (a wave's lanes run in step: what one lane wrote to prob above, another may read below)
+          if (lane < d) {
+            const float* value = v_tile + lane * 65;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int s = b * 4 + u;
+              const bool column = col_tok[s] >= run_first && col_tok[s] < run_end && col_pos[s] >= start && col_lo[s] < start + 64;
+              if (!column) continue;
+              const int first = max(0, col_lo[s] - start), last = min(64, col_pos[s] - start + 1);
+              float sum = acc[g][s];
+              for (int jj = first; jj < last; ++jj) sum += my_prob[u * 64 + jj] * value[jj];
+              acc[g][s] = sum;
+            }
+          }
+        }
+      }
+    }
+    run_first = run_end;
+  }
+  // the four states of a column into one, in their order
+  if (lane < d) {
+#pragma unroll
+    for (int s = 0; s < kTiledSlots; ++s) {
+      const int c = wave + 4 * s;
+      if (c >= ncols) continue;
+      float top = -INFINITY;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) top = fmaxf(top, run_max[g][s]);
+      float total = 0.f, result = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float m = run_max[g][s];
+        if (m == -INFINITY) continue;
+        const float w = expf(m - top);
+        total += w * run_sum[g][s];
+        result += w * acc[g][s];
+      }
+      out[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * d + lane] = from_float<T>(result / total);
+    }
+  }
+}
+
 }  // namespace tlie
 
 using namespace tlie;
@@ -124,9 +290,27 @@ using namespace tlie;
 extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtype, const int* block_table,
                                       int max_blocks, const int* token_seq, const int* positions, void* out,
                                       int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
-                                      void* stream) {
+                                      int tiled, void* stream) {
   if (tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || page_size <= 0 || max_blocks <= 0)
     return kBadArgument;
+  if (tiled && d <= 64 && (dtype == kF32 || dtype == kBF16)) {
+    // (the same bits as the kernel below, for steps whose sequences bring several tokens each)
+    const int G = nq / nkv;
+    const int heads_per_block = G < kTiledCols ? G : kTiledCols;
+    const int tokens_per_block = kTiledCols / heads_per_block;
+    const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block, nkv, (G + heads_per_block - 1) / heads_per_block);
+    const size_t bytes = (64 * static_cast<size_t>(d | 1) + static_cast<size_t>(d) * 65 + kTiledCols * static_cast<size_t>(d) + 4 * 4 * 64) *
+                         sizeof(float);
+    if (dtype == kF32)
+      hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(256), bytes, (hipStream_t)stream, (const float*)q,
+                         (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d,
+                         page_size, window, scale, tokens_per_block, heads_per_block);
+    else
+      hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(256), bytes, (hipStream_t)stream, (const bf16*)q,
+                         (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d,
+                         page_size, window, scale, tokens_per_block, heads_per_block);
+    return launch_status();
+  }
   const int chunk = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
   const int groups = 256 / chunk;
   const size_t lds = (static_cast<size_t>(d) + 256 + 4 + 2 * groups + static_cast<size_t>(groups) * d) * sizeof(float);

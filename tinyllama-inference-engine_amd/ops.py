@@ -222,9 +222,12 @@ def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, in
 
 def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, token_seq: torch.Tensor,
                       positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                      window: int | None, scale: float) -> torch.Tensor:
+                      window: int | None, scale: float, tiled: bool = False) -> torch.Tensor:
     """Causal attention of every token over its sequence's cached keys; any number of tokens per
-    sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it."""
+    sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it.
+    tiled: the step's sequences bring several tokens each (consecutive in the step, at consecutive
+    positions): neighbouring tokens then share each read of the keys (head sizes up to 64; the
+    result has the same bits either way)."""
     _device_tensor(q, "q", (torch.float32, torch.bfloat16))
     _device_tensor(cache, "cache", q.dtype)
     _device_tensor(block_table, "block_table", torch.int32)
@@ -242,7 +245,7 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     _check(library().tlie_attention_generic(_ptr(q), _ptr(cache), dtype_code(q.dtype), _ptr(block_table),
                                             block_table.shape[1], _ptr(token_seq), _ptr(positions), _ptr(out), tokens,
                                             num_heads, num_kv_heads, head_dim, page_size,
-                                            int(window) if window else 0, ctypes.c_float(scale), _stream()),
+                                            int(window) if window else 0, ctypes.c_float(scale), 1 if tiled else 0, _stream()),
            "attention_generic")
     return out
 

@@ -103,8 +103,10 @@ class Attention(Mixer):
             attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv,
                                           self.d, self.window, self.scale, nsplit, split_len, col_tiles, waves, shared)
         else:
+            # (sequences that bring four tokens or more on average: neighbouring tokens share the keys they read)
             attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
-                                             self.nkv, self.d, self.window, self.scale)
+                                             self.nkv, self.d, self.window, self.scale,
+                                             tiled=ctx.num_tokens >= 4 * ctx.num_seqs)
         return self.o(attended, into=into)
 
     def _apply_other_positions(self, qkv, ctx):
