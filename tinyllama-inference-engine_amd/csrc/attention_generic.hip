@@ -13,6 +13,8 @@
 // step was cut.
 #include "common.h"
 
+#include <type_traits>
+
 namespace tlie {
 
 // q: [tokens][nq][d]; cache: [pages][2][nkv][page_size * d], keys [row][dim], values [dim][row];
@@ -30,7 +32,7 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
                          int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                          T* __restrict__ out, int nq, int nkv, int d, int page_size, int window, float scale) {
   constexpr int kGroups = 256 / CHUNK, kWavesPerGroup = CHUNK / 64;
-  extern __shared__ float lds[];
+  extern __shared__ __attribute__((aligned(16))) float lds[];
   float* q_row = lds;                              // d
   float* prob = q_row + d;                         // 256: a group's probabilities of its current chunk
   float* wave_part = prob + 256;                   // 4: one value per wave, for the reductions within a group
@@ -49,6 +51,8 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
 
   for (int i = threadIdx.x; i < d; i += 256) q_row[i] = to_float(q[(static_cast<size_t>(t) * nq + h) * d + i]);
   __syncthreads();
+  // whole 16-byte loads of keys and values where everything is a multiple of four floats
+  const bool wide = (d & 3) == 0 && (page_size & 3) == 0 && (reinterpret_cast<uintptr_t>(cache) & 15) == 0;
 
   // the reductions over a group: over each of its waves by shuffles, then over its waves through LDS
   // (every thread of the workgroup takes part in every call: the barriers are the workgroup's)
@@ -74,7 +78,20 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
       const T* key = cache + static_cast<size_t>(pages[j / page_size]) * page_stride + head_offset +
                      static_cast<size_t>(j % page_size) * d;
       float dot = 0.f;
-      for (int i = 0; i < d; ++i) dot += q_row[i] * to_float(key[i]);
+      int i = 0;
+      if (std::is_same<T, float>::value && wide) {
+        // (four dims a load; the additions stay in the order of the dims)
+#pragma unroll 4
+        for (; i + 4 <= d; i += 4) {
+          const float4 kv = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(key) + i);
+          const float4 qv = *reinterpret_cast<const float4*>(q_row + i);
+          dot += qv.x * kv.x;
+          dot += qv.y * kv.y;
+          dot += qv.z * kv.z;
+          dot += qv.w * kv.w;
+        }
+      }
+      for (; i < d; ++i) dot += q_row[i] * to_float(key[i]);
       score = dot * scale;
     }
     const float new_max = fmaxf(running_max, over_group(score, true));
@@ -89,7 +106,30 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
     if (place < d) {
       acc *= alpha;
       const int first = max(0, lo - start), last = min(CHUNK, pos - start + 1);
-      for (int jj = first; jj < last; ++jj) {
+      int jj = first;
+      if (std::is_same<T, float>::value && wide) {
+        // (four keys a load where they lie on one page, four to a boundary: chunks start at multiples of
+        // 64 and pages hold a multiple of four rows; the additions stay in the order of the keys)
+        for (; jj < last && (jj & 3) != 0; ++jj) {
+          const int key_pos = start + jj;
+          const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset + head_offset +
+                           static_cast<size_t>(place) * page_size + key_pos % page_size;
+          acc += prob[group * CHUNK + jj] * to_float(*value);
+        }
+#pragma unroll 4
+        for (; jj + 4 <= last; jj += 4) {
+          const int key_pos = start + jj;
+          const float* value = reinterpret_cast<const float*>(cache) + static_cast<size_t>(pages[key_pos / page_size]) * page_stride +
+                               v_offset + head_offset + static_cast<size_t>(place) * page_size + key_pos % page_size;
+          const float4 vv = *reinterpret_cast<const float4*>(value);
+          const float4 pv = *reinterpret_cast<const float4*>(prob + group * CHUNK + jj);
+          acc += pv.x * vv.x;
+          acc += pv.y * vv.y;
+          acc += pv.z * vv.z;
+          acc += pv.w * vv.w;
+        }
+      }
+      for (; jj < last; ++jj) {
         const int key_pos = start + jj;
         const T* value = cache + static_cast<size_t>(pages[key_pos / page_size]) * page_stride + v_offset + head_offset +
                          static_cast<size_t>(place) * page_size + key_pos % page_size;
@@ -130,19 +170,22 @@ attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, c
 // A column therefore gets the same bits from either kernel, and a step may take whichever is faster.
 // Head sizes up to 64.  Tokens of a workgroup that belong to different sequences are served one
 // run of equal sequences after the other.
-constexpr int kTiledCols = 32, kTiledSlots = 8;     // columns a workgroup, columns a wave
+constexpr int kTiledCols = 32, kTiledWaves = 8, kTiledSlots = kTiledCols / kTiledWaves;     // columns a workgroup, its waves, columns a wave
 template <typename T>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64 * kTiledWaves)
 attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                                int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                                T* __restrict__ out, int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
                                int tokens_per_block, int heads_per_block) {
-  extern __shared__ float lds[];
-  const int k_stride = d | 1;                      // odd: the 64 lanes of a wave read 64 different banks
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // rows of a multiple of 4 floats, so that four values are one LDS read, plus 4: a wave's lanes, each
+  // on a row of its own, then spread over the banks
+  const int k_stride = (d + 3) / 4 * 4 + 4, q_stride = (d + 3) / 4 * 4;
+  constexpr int kValueStride = 68;
   float* k_tile = lds;                             // [64 keys][k_stride]
-  float* v_tile = k_tile + 64 * k_stride;          // [d][65]
-  float* q_tile = v_tile + d * 65;                 // [32 columns][d]
-  float* prob = q_tile + kTiledCols * d;           // [4 waves][4 columns][64 keys]
+  float* v_tile = k_tile + 64 * k_stride;          // [d][68]
+  float* q_tile = v_tile + d * kValueStride;       // [32 columns][q_stride]
+  float* prob = q_tile + kTiledCols * q_stride;    // [waves][4 columns][64 keys]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int G = nq / nkv, kv_head = blockIdx.y;
   const int tok0 = blockIdx.x * tokens_per_block, head0 = blockIdx.z * heads_per_block;
@@ -152,15 +195,15 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
   const size_t head_offset = static_cast<size_t>(kv_head) * page_size * d;
   const size_t v_offset = static_cast<size_t>(nkv) * page_size * d;
 
-  for (int e = threadIdx.x; e < ncols * d; e += 256) {
+  for (int e = threadIdx.x; e < ncols * d; e += 64 * kTiledWaves) {
     const int c = e / d, i = e - c * d;
-    q_tile[c * d + i] = to_float(q[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * d + i]);
+    q_tile[c * q_stride + i] = to_float(q[(static_cast<size_t>(tok0 + c / nheads) * nq + kv_head * G + head0 + c % nheads) * d + i]);
   }
-  // this wave's columns: slot s is column wave + 4 s
+  // this wave's columns: slot s is column wave + kTiledWaves * s
   int col_pos[kTiledSlots], col_lo[kTiledSlots], col_tok[kTiledSlots];     // col_tok: the column's token among the workgroup's, or -1
 #pragma unroll
   for (int s = 0; s < kTiledSlots; ++s) {
-    const int c = wave + 4 * s;
+    const int c = wave + kTiledWaves * s;
     const bool live = c < ncols;
     col_tok[s] = live ? c / nheads : -1;
     col_pos[s] = live ? positions[tok0 + col_tok[s]] : -1;
@@ -194,16 +237,16 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
         const int start = base + g * 64;
         if (start > hi) break;                     // (uniform)
         __syncthreads();                           // the tiles of the chunk before have been read
-        for (int e = threadIdx.x; e < 64 * d; e += 256) {
+        for (int e = threadIdx.x; e < 64 * d; e += 64 * kTiledWaves) {
           const int r = e / d, i = e - r * d, j = start + r;
           if (j <= hi && j >= lo)
             k_tile[r * k_stride + i] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + head_offset +
                                                       static_cast<size_t>(j % page_size) * d + i]);
         }
-        for (int e = threadIdx.x; e < 64 * d; e += 256) {
+        for (int e = threadIdx.x; e < 64 * d; e += 64 * kTiledWaves) {
           const int dim = e >> 6, r = e & 63, j = start + r;
           if (j <= hi && j >= lo)
-            v_tile[dim * 65 + r] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + v_offset + head_offset +
+            v_tile[dim * kValueStride + r] = to_float(cache[static_cast<size_t>(pages[j / page_size]) * page_stride + v_offset + head_offset +
                                                   static_cast<size_t>(dim) * page_size + j % page_size]);
         }
         __syncthreads();
@@ -219,10 +262,27 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
           const int j = start + lane;
           float dot[4] = {0.f, 0.f, 0.f, 0.f};
           const float* key = k_tile + lane * k_stride;
-          for (int i = 0; i < d; ++i) {
+          const float* query[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) query[u] = q_tile + min(wave + kTiledWaves * (b * 4 + u), kTiledCols - 1) * q_stride;
+          // (four dims a read; the additions of a column stay in the order of the dims)
+          int i = 0;
+#pragma unroll 4
+          for (; i + 4 <= d; i += 4) {
+            const float4 kv = *reinterpret_cast<const float4*>(key + i);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const float4 qv = *reinterpret_cast<const float4*>(query[u] + i);
+              dot[u] += qv.x * kv.x;
+              dot[u] += qv.y * kv.y;
+              dot[u] += qv.z * kv.z;
+              dot[u] += qv.w * kv.w;
+            }
+          }
+          for (; i < d; ++i) {
             const float kv = key[i];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) dot[u] += q_tile[min(wave + 4 * (b * 4 + u), kTiledCols - 1) * d + i] * kv;
+            for (int u = 0; u < 4; ++u) dot[u] += query[u][i] * kv;
           }
           float* my_prob = prob + (wave * 4) * 64;
 #pragma unroll
@@ -243,7 +303,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
           }
           // (a wave's lanes run in step: what one lane wrote to prob above, another may read below)
           if (lane < d) {
-            const float* value = v_tile + lane * 65;
+            const float* value = v_tile + lane * kValueStride;
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
               const int s = b * 4 + u;
@@ -251,7 +311,18 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
               if (!column) continue;
               const int first = max(0, col_lo[s] - start), last = min(64, col_pos[s] - start + 1);
               float sum = acc[g][s];
-              for (int jj = first; jj < last; ++jj) sum += my_prob[u * 64 + jj] * value[jj];
+              const float* weight = my_prob + u * 64;
+              int jj = first;
+              for (; jj < last && (jj & 3) != 0; ++jj) sum += weight[jj] * value[jj];
+#pragma unroll 4
+              for (; jj + 4 <= last; jj += 4) {           // (four keys a read; the additions stay in the order of the keys)
+                const float4 pv = *reinterpret_cast<const float4*>(weight + jj), vv = *reinterpret_cast<const float4*>(value + jj);
+                sum += pv.x * vv.x;
+                sum += pv.y * vv.y;
+                sum += pv.z * vv.z;
+                sum += pv.w * vv.w;
+              }
+              for (; jj < last; ++jj) sum += weight[jj] * value[jj];
               acc[g][s] = sum;
             }
           }
@@ -264,7 +335,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
   if (lane < d) {
 #pragma unroll
     for (int s = 0; s < kTiledSlots; ++s) {
-      const int c = wave + 4 * s;
+      const int c = wave + kTiledWaves * s;
       if (c >= ncols) continue;
       float top = -INFINITY;
 #pragma unroll
@@ -299,14 +370,14 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
     const int heads_per_block = G < kTiledCols ? G : kTiledCols;
     const int tokens_per_block = kTiledCols / heads_per_block;
     const dim3 grid((tokens + tokens_per_block - 1) / tokens_per_block, nkv, (G + heads_per_block - 1) / heads_per_block);
-    const size_t bytes = (64 * static_cast<size_t>(d | 1) + static_cast<size_t>(d) * 65 + kTiledCols * static_cast<size_t>(d) + 4 * 4 * 64) *
-                         sizeof(float);
+    const size_t rounded = (static_cast<size_t>(d) + 3) / 4 * 4;
+    const size_t bytes = (64 * (rounded + 4) + static_cast<size_t>(d) * 68 + kTiledCols * rounded + kTiledWaves * 4 * 64) * sizeof(float);
     if (dtype == kF32)
-      hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(256), bytes, (hipStream_t)stream, (const float*)q,
+      hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const float*)q,
                          (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d,
                          page_size, window, scale, tokens_per_block, heads_per_block);
     else
-      hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(256), bytes, (hipStream_t)stream, (const bf16*)q,
+      hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const bf16*)q,
                          (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d,
                          page_size, window, scale, tokens_per_block, heads_per_block);
     return launch_status();
