@@ -399,6 +399,37 @@ def test_gemm_skinny(shape):
         assert torch.equal(alone[:, 0], together[:, 0])                      # every partial sum, bit for bit
 
 
+@pytest.mark.parametrize("rows", [5, 23, 40, 64])
+def test_gemm_skinny_launch_shapes(rows):
+    """Every number of waves a workgroup and both numbers of strips a wave give the same partial
+    sums, bit for bit (the shape decides who computes an output, not how), at sizes where the last
+    workgroup and the last split are ragged; and the shape that the policy picks is one of them."""
+    from tlie_amd import ops
+    n, k = 1000, 840                                          # 1000 = 62.5 strips; 840 = 3 splits of 320, the last of 200
+    torch.manual_seed(rows)
+    x = torch.randn(rows, k).bfloat16().to(DEV)
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16().to(DEV)
+    b = torch.randn(n).bfloat16().to(DEV)
+    first = ops.gemm_skinny(x, w, b, split_len=320, waves=4, strips=1)
+    assert first.nsplit == 3
+    assert rel_err(first.dense().cpu(), plain_linear(x.cpu().double(), w.cpu().double(), b.cpu().double())) < 5e-6
+    for waves in range(4, 17):
+        for strips in (1, 2):
+            if strips == 2 and (rows <= 32 or waves > 8):
+                with pytest.raises(ops.EngineError):
+                    ops.gemm_skinny(x, w, b, split_len=320, waves=waves, strips=strips)
+                continue
+            other = ops.gemm_skinny(x, w, b, split_len=320, waves=waves, strips=strips)
+            assert torch.equal(other.data, first.data), (waves, strips)
+    split_len, waves, strips = ops.skinny_plan(rows, n, k, 256)
+    planned = ops.gemm_skinny(x, w, b)
+    assert planned.nsplit == (k + split_len - 1) // split_len and 4 <= waves <= 16 and strips in (1, 2)
+    assert rel_err(planned.dense().cpu(), plain_linear(x.cpu().double(), w.cpu().double(), b.cpu().double())) < 5e-6
+    for bad in (dict(waves=3), dict(waves=17), dict(strips=3)):
+        with pytest.raises(ops.EngineError):
+            ops.gemm_skinny(x, w, b, split_len=320, **{"waves": 4, "strips": 1, **bad})
+
+
 def test_gemm_skinny_refuses():
     from tlie_amd import EngineError, ops
     w = torch.randn(32, 64, device=DEV).bfloat16()

@@ -49,3 +49,25 @@ def test_what_no_recording_serves():
     assert made.records([StepEntry(0, [0], [0], source=3), StepEntry(1, [1, 2], [1])]) is None
     made.use_graphs = False
     assert made.records(entries([5, 3])) is None and not made.replays(entries([1]))
+
+
+def test_the_skinny_products_launch_shape_is_one_the_kernel_takes():
+    """Decided on the host from the sizes alone: every plan is within what the kernel takes, covers
+    the inner size exactly, and for matrices that the policy balances the workgroups are no more
+    than the compute units (one round) unless a round more is cheaper than more splits."""
+    from tlie_amd import ops
+    for rows in (1, 16, 17, 32, 33, 64):
+        for out_features, in_features in ((2560, 2048), (2048, 2048), (11264, 2048), (2048, 5632), (32000, 2048), (100, 520),
+                                          (515, 1000), (64, 5632), (12288, 4096), (28672, 4096), (4096, 14336), (7, 8)):
+            for units in (256, 304, 64):
+                split_len, waves, strips = ops.skinny_plan(rows, out_features, in_features, units)
+                assert split_len > 0 and split_len % 64 == 0 and 4 <= waves <= 16 and strips in (1, 2)
+                assert strips == 1 or (rows > 32 and waves <= 8)
+                nsplit = -(-in_features // split_len)
+                assert (nsplit - 1) * split_len < in_features <= nsplit * split_len
+                assert ops.skinny_plan(rows, out_features, in_features, units) == (split_len, waves, strips)    # (kept)
+    # TinyLlama's four matrices at 64 rows on 256 compute units: one round of workgroups
+    for out_features, in_features in ((2560, 2048), (2048, 2048), (11264, 2048), (2048, 5632)):
+        split_len, waves, strips = ops.skinny_plan(64, out_features, in_features, 256)
+        workgroups = -(-out_features // (16 * waves * strips)) * -(-in_features // split_len)
+        assert 128 < workgroups <= 256, (out_features, in_features, split_len, waves, strips)

@@ -91,9 +91,13 @@ constexpr int attention_max_waves(int dt, int ct) {
 // SHARED: the waves of a workgroup do not share a tile's keys but take 16 * CT columns each of a
 // tile of 16 * CT * waves columns, and every block of keys and values is brought once, through LDS,
 // for all of them (prompt portions: the tiles of neighbouring tokens read the same keys, and read
-// each on its own they are bound by the L2's bandwidth, not by their arithmetic).
+// each on its own they are bound by the L2's bandwidth, not by their arithmetic).  These kernels
+// wait more than they compute (a block's chain of loads, products, maxima and exponentials is
+// longer than what a wave can issue meanwhile), so for head sizes up to 64 the compiler is asked to
+// stay within the registers of 4 waves a SIMD with one column group and 3 with two, where it would
+// take those of 3 and 2 (a prompt of 2048 tokens 53 -> 51 us, of 4096 158 -> 150).
 template <int DT, int CT, bool SHARED>
-__global__ void __launch_bounds__(SHARED ? 512 : 64 * attention_max_waves(DT, CT))
+__global__ void __launch_bounds__(SHARED ? 512 : 64 * attention_max_waves(DT, CT), (SHARED && DT <= 4) ? (CT == 1 ? 4 : 3) : 1)
 attention_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ cache,
                       const int* __restrict__ block_table, int max_blocks, const int4* __restrict__ tiles,
                       const int* __restrict__ positions, uint16_t* __restrict__ out, float* __restrict__ part_o,

@@ -26,15 +26,18 @@ union Pack16 {
   bf16x8 v;
 };
 
-constexpr int kSkinnyThreads = 256;          // 4 waves
 constexpr int kSkinnyPad = 8;                // bf16 elements of padding per LDS row (16 bytes): rows fall on different banks
 
-// NT: tiles of 16 rows of x (M <= 16 * NT).  RS: strips of 16 rows of W per wave (a block takes
-// 64 * RS rows): with more rows of x, more strips share each read of x from LDS and each staging of
-// x from global memory.  CHUNK: k values staged in LDS at a time.
+// NT: tiles of 16 rows of x (M <= 16 * NT).  RS: strips of 16 rows of W per wave: with more rows
+// of x, more strips share each read of x from LDS.  A workgroup has blockDim.x / 64 waves, at most
+// MAXWAVES and at least MINWAVES, and takes 16 * RS rows of W per wave: the caller picks the number of waves and the
+// split's length so that the workgroups are as many as the compute units, or a multiple (a compute
+// unit draws some 20 GB/s from memory whatever its waves ask for, so the product takes as long as
+// the unit with the most bytes; 176 workgroups on 256 units measured 3.1 TB/s, 256 of them 4.3).
+// CHUNK: k values staged in LDS at a time.
 // split_len: k values per split (multiple of 64).  K % 8 == 0.
-template <int NT, int RS, int CHUNK>
-__global__ void __launch_bounds__(kSkinnyThreads)
+template <int NT, int RS, int CHUNK, int MINWAVES, int MAXWAVES>
+__global__ void __launch_bounds__(64 * MAXWAVES)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
                    float* __restrict__ y, int M, int N, int K, int split_len) {
   constexpr int kStride = CHUNK + kSkinnyPad;
@@ -43,7 +46,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int split = blockIdx.y;
   const int k_begin = split * split_len, k_end = min(K, k_begin + split_len);
-  const int wave_row = (blockIdx.x * 4 + wave) * 16 * RS;
+  const int wave_row = (blockIdx.x * (blockDim.x >> 6) + wave) * 16 * RS;
   const int group = lane >> 4;
   const uint16_t* w_row[RS];
   bool active[RS];
@@ -62,7 +65,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   // Two sets of operand registers in turn: the next chunk's part of W, and its part of x, are asked
   // for before the current chunk is multiplied, so that memory and the matrix cores work at once.
   constexpr int kVectors = CHUNK / 8;                                  // 16-byte pieces of a staged row of x
-  constexpr int kStage = (NT * 16 * kVectors + kSkinnyThreads - 1) / kSkinnyThreads;   // pieces a thread stages
+  constexpr int kStage = (NT * 16 * kVectors + 64 * MINWAVES - 1) / (64 * MINWAVES);   // pieces a thread stages
   Pack16 a[2][RS][kSteps][2];
   uint4 staged[kStage];
   auto load_w = [&](int c0, Pack16 (&buf)[RS][kSteps][2]) {
@@ -80,7 +83,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
     const int c1 = min(k_end, c0 + CHUNK);
 #pragma unroll
     for (int j = 0; j < kStage; ++j) {
-      const int i = threadIdx.x + j * kSkinnyThreads;
+      const int i = threadIdx.x + j * blockDim.x;
       const int token = i / kVectors, k = c0 + (i % kVectors) * 8;
       staged[j] = (token < M && k < c1) ? *reinterpret_cast<const uint4*>(x + static_cast<size_t>(token) * K + k)
                                         : make_uint4(0, 0, 0, 0);
@@ -89,7 +92,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
   auto store_x = [&]() {
 #pragma unroll
     for (int j = 0; j < kStage; ++j) {
-      const int i = threadIdx.x + j * kSkinnyThreads;
+      const int i = threadIdx.x + j * blockDim.x;
       if (i < NT * 16 * kVectors) *reinterpret_cast<uint4*>(xs + (i / kVectors) * kStride + (i % kVectors) * 8) = staged[j];
     }
   };
@@ -162,26 +165,49 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
 
 using namespace tlie;
 
+namespace {
+
+template <int NT, int RS>
+int launch_skinny(dim3 grid, int waves, hipStream_t s, const uint16_t* x, const uint16_t* w, const uint16_t* bias, float* y, int M,
+                  int N, int K, int split_len) {
+  // (the staged chunk is as long as the registers allow for the workgroup's size)
+  const dim3 block(64 * waves);
+  if (waves <= 4) {
+    constexpr int kChunk = NT <= 2 ? 512 : 256;
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 4, 4>), grid, block, 0, s, x, w, bias, y, M, N, K, split_len);
+  } else if (waves <= 8) {
+    constexpr int kChunk = RS == 1 ? 256 : 128;
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 5, 8>), grid, block, 0, s, x, w, bias, y, M, N, K, split_len);
+  } else {
+    if constexpr (RS == 1)
+      hipLaunchKernelGGL((gemm_skinny_kernel<NT, 1, (NT <= 2 ? 256 : 128), 9, 16>), grid, block, 0, s, x, w, bias, y, M, N, K, split_len);
+    else
+      return kBadArgument;
+  }
+  return launch_status();
+}
+
+}  // namespace
+
 // x [M, K], w [N, K], bias [N] or null: bfloat16.  y: float [nsplit, M, N] with
 // nsplit = ceil(K / split_len).  M <= 64, K % 8 == 0, split_len % 64 == 0.
+// waves: 4 to 16 waves a workgroup; strips: 1 or 2 strips of 16 rows of W per wave (2 only for more
+// than 32 rows of x and up to 8 waves); a workgroup takes 16 * strips * waves rows of W.
 extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, float* y, int M, int N, int K,
-                                int split_len, void* stream) {
+                                int split_len, int waves, int strips, void* stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) != 0 || split_len <= 0 || (split_len & 63) != 0) return kBadArgument;
+  if (waves < 4 || waves > 16 || strips < 1 || strips > 2 || (strips == 2 && (M <= 32 || waves > 8))) return kBadArgument;
   const int nsplit = (K + split_len - 1) / split_len;
   const int tiles = (M + 15) / 16;
-  const int nt = tiles <= 1 ? 1 : (tiles == 2 ? 2 : 4);
-  const int rows_per_block = nt == 4 ? 128 : 64;
+  const int rows_per_block = 16 * strips * waves;
   const dim3 grid((N + rows_per_block - 1) / rows_per_block, nsplit);
   if (grid.y > 65535) return kBadArgument;
   hipStream_t s = (hipStream_t)stream;
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (nt == 1)
-    hipLaunchKernelGGL((gemm_skinny_kernel<1, 1, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
-  else if (nt == 2)
-    hipLaunchKernelGGL((gemm_skinny_kernel<2, 1, 512>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
-  else
-    hipLaunchKernelGGL((gemm_skinny_kernel<4, 2, 256>), grid, dim3(kSkinnyThreads), 0, s, xp, wp, bp, y, M, N, K, split_len);
-  return launch_status();
+  if (tiles <= 1) return launch_skinny<1, 1>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
+  if (tiles == 2) return launch_skinny<2, 1>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
+  if (strips == 1) return launch_skinny<4, 1>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
+  return launch_skinny<4, 2>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
 }

@@ -377,12 +377,11 @@ def feed_tokens(tokens: torch.Tensor, source: torch.Tensor, sampled: torch.Tenso
 # ---- bfloat16 kernels on the matrix cores ---------------------------------------------------------
 SKINNY_MAX_ROWS = 64
 def skinny_split_len(rows: int, out_features: int, in_features: int) -> int:
-    """How many k values one split takes.  Measured on the MI355X inside whole decode steps of the
-    TinyLlama shapes: matrices of few rows (2048, 2560) are fastest with 256 k values a workgroup
-    (longer splits leave the 256 CUs too few workgroups); the gated feed-forward's first product
-    (11264 rows) with 512, and 1024 once the step has more than 32 rows of x, because each partial
-    sum is a write and a read of rows x outputs; a long inner size (5632) with 1024 up to 32 rows
-    and 512 beyond."""
+    """How many k values one split takes when the matrix has work for many workgroups per compute
+    unit.  Measured on the MI355X inside whole decode steps: the gated feed-forward's first product
+    (11264 rows and more) with 512, and 1024 once the step has more than 32 rows of x, because each
+    partial sum is a write and a read of rows x outputs; a long inner size (4096 and more) with 1024
+    up to 32 rows and 512 beyond; the others with 256."""
     strips = (out_features + 15) // 16
     if strips >= 512:
         length = 1024 if rows > 32 else 512
@@ -393,13 +392,59 @@ def skinny_split_len(rows: int, out_features: int, in_features: int) -> int:
     return min(length, (in_features + 63) // 64 * 64)
 
 
+_SKINNY_PLANS: dict = {}
+_COMPUTE_UNITS: dict = {}
+
+
+def _compute_units(device: torch.device) -> int:
+    index = device.index or 0
+    if index not in _COMPUTE_UNITS:
+        _COMPUTE_UNITS[index] = int(torch.cuda.get_device_properties(device).multi_processor_count)
+    return _COMPUTE_UNITS[index]
+
+
+def skinny_plan(rows: int, out_features: int, in_features: int, compute_units: int = 256) -> tuple[int, int, int]:
+    """The launch shape of `gemm_skinny`: (k values per split, waves a workgroup, strips of 16 rows
+    of W a wave).  A compute unit draws some 20 GB/s from memory whatever its waves ask for, so a
+    matrix of up to 64 MB is cut into as many equal workgroups as there are compute units, or just
+    fewer (the product takes as long as the unit with the most bytes: TinyLlama's q/k/v matrix at 64
+    rows 7.4 -> 6.4 us, the output projection 6.9 -> 5.7, gate/up 17.9 -> 16.9, down 11.0 -> 10.3),
+    by the number of waves (each takes 16 rows of W) and the number of splits, each split costing a
+    write and a read of rows x outputs partial sums (a decode step of the TinyLlama shape at batch
+    64 2.10 -> 2.01 ms, at 32 1.69 -> 1.63).  Larger matrices keep many workgroups per compute unit
+    (several at once hide each other's waits, which counts for more there)."""
+    key = (rows, out_features, in_features, compute_units)
+    if key in _SKINNY_PLANS:
+        return _SKINNY_PLANS[key]
+    plan = (skinny_split_len(rows, out_features, in_features), 4, 2 if rows > 32 else 1)
+    if out_features * in_features * 2 <= (64 << 20):
+        best = None
+        for waves in range(4, 17):
+            blocks = -(-out_features // (16 * waves))
+            for nsplit in range(1, 33):
+                split_len = (-(-in_features // nsplit) + 63) // 64 * 64
+                if -(-in_features // split_len) != nsplit:
+                    continue
+                rounds = -(-blocks * nsplit // compute_units)
+                # microseconds: a workgroup's bytes at 20 GB/s and half a microsecond per round; the partial sums at 6 TB/s
+                # (the coefficients that gave the fastest whole decode steps at 20, 32 and 64 rows)
+                cost = rounds * (16 * waves * split_len * 2 / 20e3 + 0.5) + nsplit * rows * out_features * 8 / 6e6
+                if best is None or cost < best[0]:
+                    best = (cost, split_len, waves, 1)
+        plan = best[1:]
+    _SKINNY_PLANS[key] = plan
+    return plan
+
+
 def gemm_skinny_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
     return (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < x.shape[0] <= SKINNY_MAX_ROWS
             and weight.shape[1] % 8 == 0)
 
 
-def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, split_len: int | None = None) -> Product:
-    """y = x . W^T (+ bias) for at most 64 rows of bfloat16 x: float partial sums [nsplit, M, N]."""
+def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, split_len: int | None = None,
+                waves: int | None = None, strips: int | None = None) -> Product:
+    """y = x . W^T (+ bias) for at most 64 rows of bfloat16 x: float partial sums [nsplit, M, N].
+    split_len, waves, strips: the launch shape (see `skinny_plan`, which chooses it when they are not given)."""
     _device_tensor(x, "x", torch.bfloat16)
     _device_tensor(weight, "weight", torch.bfloat16)
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -411,13 +456,18 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None
         _device_tensor(bias, "bias", torch.bfloat16)
         if bias.shape != (out_features,):
             raise invalid_shape("gemm_skinny: bias needs one entry per output")
-    split_len = split_len or skinny_split_len(rows, out_features, in_features)
+    if split_len is None:
+        split_len, waves, strips = skinny_plan(rows, out_features, in_features, _compute_units(x.device))
+    elif waves is None or strips is None:
+        waves, strips = waves or 4, strips or (2 if rows > 32 else 1)
     if split_len <= 0 or split_len % 64 != 0:
         raise invalid_argument("gemm_skinny: a split's length must be a positive multiple of 64")
+    if not 4 <= waves <= 16 or strips not in (1, 2) or (strips == 2 and (rows <= 32 or waves > 8)):
+        raise invalid_argument("gemm_skinny: 4 to 16 waves; two strips a wave only for more than 32 rows and up to 8 waves")
     nsplit = (in_features + split_len - 1) // split_len
     out = torch.empty((nsplit, rows, out_features), dtype=torch.float32, device=x.device)
     _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), rows, out_features, in_features,
-                                      split_len, _stream()), "gemm_skinny")
+                                      split_len, waves, strips, _stream()), "gemm_skinny")
     return Product(out, nsplit)
 
 
@@ -482,10 +532,11 @@ def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
         col_tiles = attention_col_tiles(head_dim)
         # sequences of some length with portions of many columns: 4 waves take columns of their own
         # of one tile and every block of keys is brought once for all of them, through LDS (a
-        # prompt of 1536 tokens: 34 us against 42; of 8192: 500 against 780; of 512: 15 against
-        # 13).  Each wave takes 32 columns, or 16 while that leaves no more tiles than two for
-        # every compute unit: they are then all at work at once, and smaller ones fill the chip
-        # better (1024 tokens: 24 us against 30; from 3072 on the larger tiles win)
+        # prompt of 1536 tokens: 34 us against 42; of 8192: 450 against 780; of 512: 15 against
+        # 13).  Each wave takes 32 columns, or 16 while that leaves no more tiles than two and a
+        # half for every compute unit: the smaller ones then fill the chip better, four
+        # workgroups a compute unit (2048 tokens: 51 us against 63; 2560: 74 against 81; 3072:
+        # 100 against 98; 4096: 162 against 150)
         shared = (col_tiles == 2 and head_dim <= 128 and ctx.max_context >= 768
                   and ctx.num_tokens * groups_per_kv >= 64 * ctx.num_seqs)
 
@@ -502,7 +553,7 @@ def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
                     ctx.scratch[key] = torch.from_numpy(make(ctx.host)).to(ctx.tokens.device)
             return ctx.scratch[key]
         tiles = tiles_of(col_tiles * (4 if shared else 1))
-        if shared and tiles.shape[0] * num_kv_heads <= 2 * ctx.compute_units:
+        if shared and 2 * tiles.shape[0] * num_kv_heads <= 5 * ctx.compute_units:
             col_tiles = 1
             tiles = tiles_of(4)
         count = tiles.shape[0] * (4 if shared else 1)
