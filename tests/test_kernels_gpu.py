@@ -430,6 +430,26 @@ def test_gemm_skinny_launch_shapes(rows):
             ops.gemm_skinny(x, w, b, split_len=320, **{"waves": 4, "strips": 1, **bad})
 
 
+@pytest.mark.parametrize("shape", [(15832, 2560, 2048), (40000, 2048, 5632), (70000, 704, 512), (65, 96, 64), (300, 32000, 256)])
+def test_library_mm_takes_the_library_for_many_rows(shape):
+    """Steps of very many rows (all prompts of a batch in one step) still go through the vendor's
+    library: its first choice for some of these shapes wants more workspace than is there, and the
+    product then takes the first candidate that fits, not the plain kernel (ten times slower)."""
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(m)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).bfloat16()
+    before = ops.library_fallbacks()
+    got = ops.library_mm(x, w)
+    got32 = ops.library_mm(x[:70], w, torch.float32)
+    assert ops.library_fallbacks() == before
+    rows = torch.tensor([0, 1, m // 2, m - 1], device=DEV)
+    want = x[rows].double() @ w.double().t()
+    assert rel_err(got[rows].cpu(), want.cpu()) < 6e-3                       # one rounding to bfloat16
+    assert rel_err(got32[:2].cpu(), want[:2].cpu()) < 5e-5
+
+
 def test_gemm_skinny_refuses():
     from tlie_amd import EngineError, ops
     w = torch.randn(32, 64, device=DEV).bfloat16()

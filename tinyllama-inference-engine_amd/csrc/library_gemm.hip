@@ -6,7 +6,7 @@
 // layer; this file calls the same library function itself, with the matrix layouts and the
 // algorithm it chose kept per shape, for 10 us.  The library is the copy that torch has loaded
 // (its functions are looked up in that file at run time, so nothing here links against a second
-// copy); the algorithm is the library's own first choice, which is also what torch takes.
+// copy); the algorithm is the library's own first choice among those that fit the workspace.
 #include "common.h"
 
 #include <dlfcn.h>
@@ -116,11 +116,18 @@ extern "C" int tlie_library_gemm(const void* x, const void* w, void* y, int y_fl
                 api.preference_set(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &workspace_bytes,
                                    sizeof(workspace_bytes)) == HIPBLAS_STATUS_SUCCESS;
     if (made) {
-      hipblasLtMatmulHeuristicResult_t result[1];
-      int returned = 0;
-      made = api.heuristic(handle->second, plan.desc, plan.w, plan.x, plan.y, plan.y, preference, 1, result, &returned) ==
-                 HIPBLAS_STATUS_SUCCESS && returned >= 1 && result[0].workspaceSize <= workspace_bytes;
-      if (made) plan.algo = result[0].algo;
+      // the library's candidates come best first by its own estimate; the first one that works
+      // within the caller's workspace is taken (for some shapes of very many rows its first
+      // choice wants more than any fixed workspace holds)
+      constexpr int kCandidates = 16;
+      hipblasLtMatmulHeuristicResult_t result[kCandidates];
+      int returned = 0, chosen = -1;
+      made = api.heuristic(handle->second, plan.desc, plan.w, plan.x, plan.y, plan.y, preference, kCandidates, result,
+                           &returned) == HIPBLAS_STATUS_SUCCESS;
+      for (int i = 0; made && chosen < 0 && i < returned; ++i)
+        if (result[i].state == HIPBLAS_STATUS_SUCCESS && result[i].workspaceSize <= workspace_bytes) chosen = i;
+      made = made && chosen >= 0;
+      if (made) plan.algo = result[chosen].algo;
     }
     if (preference != nullptr) api.preference_destroy(preference);
     plan.usable = made;                 // (a shape without an algorithm is remembered too, and not asked for again)

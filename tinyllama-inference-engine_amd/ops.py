@@ -269,7 +269,8 @@ def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | Non
     return Product(out, 1)
 
 
-_library_gemm = {"state": None, "workspace": {}}       # state: None (not tried), True, False (not there)
+# state: None (not tried), True, False (not there); fallbacks: products that took this library's plain kernel instead
+_library_gemm = {"state": None, "workspace": {}, "fallbacks": 0}
 LIBRARY_WORKSPACE_BYTES = 32 << 20
 
 
@@ -309,7 +310,15 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
     # algorithm for the shape) this library's plain kernel makes the product: one route, recorded or
     # not, so that a step gives the same bits replayed and launched (slow, and safe inside a recording,
     # where a library call that has not been tried may clear a workspace with a memset node)
+    if x.shape[0] > 0:
+        state["fallbacks"] += 1
     return gemm_generic(x, weight, None, out_dtype).data
+
+
+def library_fallbacks() -> int:
+    """How many products `library_mm` has made with the plain kernel because the vendor's library
+    was not there or offered nothing for the shape (each many times slower)."""
+    return _library_gemm["fallbacks"]
 
 
 def add_bias(product: torch.Tensor, bias: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
