@@ -668,7 +668,7 @@ def test_gemm_rows(shape):
     got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV)).dense()
     assert got.dtype == torch.float32 and rel_err(got, want) < 5e-6
     for waves in (2, 4, 8, 16):
-        for rows_per_block in (8, 16, 32):
+        for rows_per_block in (2, 6, 8, 10, 12, 16, 32):
             if rows_per_block == 32 and waves == 16:
                 with pytest.raises(ops.EngineError):
                     ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), waves=waves, rows_per_block=rows_per_block)
@@ -692,7 +692,7 @@ def test_gemm_rows(shape):
     if n % 2 == 0:
         # rows of W alternate gate and up
         full = plain_linear(x.double(), w.double())
-        for rows_per_block, waves in ((8, None), (16, None), (32, 4), (32, 2), (16, 2)):
+        for rows_per_block, waves in ((8, None), (16, None), (32, 4), (32, 2), (16, 2), (10, None), (6, 16)):
             act = ops.gemm_rows(x.to(DEV), w.to(DEV), None, "silu", rows_per_block=rows_per_block, waves=waves)
             assert act.shape == (m, n // 2) and rel_err(act, plain_silu_mul(full[:, 0::2], full[:, 1::2])) < TOL["bfloat16"]
         # the same layout through the kernel that adds up partial sums
@@ -701,7 +701,7 @@ def test_gemm_rows(shape):
     # added into the residual, with the next norm's inputs
     target = torch.randn(m, n)
     next_g = (1 + 0.2 * torch.randn(n)).bfloat16()
-    for next_weight, rows_per_block in ((next_g, 16), (next_g.float(), 8), (next_g, 32)):
+    for next_weight, rows_per_block in ((next_g, 16), (next_g.float(), 8), (next_g, 32), (next_g, 10)):
         res_dev = target.clone().to(DEV)
         updated = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), "residual", residual=res_dev,
                                 next_norm=(next_weight.to(DEV), 1e-6), rows_per_block=rows_per_block,
@@ -770,7 +770,7 @@ def test_rotation_in_paired_order_and_inside_the_product(case):
     paired_q = ops.rope_cache(ops.gemm_skinny(x, w_paired, b_paired), positions, slots, inv_freq, rot, paired_cache, nq, nkv, d,
                               torch.bfloat16, paired=True)
     assert torch.equal(paired_q, plain_q) and torch.equal(paired_cache, plain_cache)
-    for rows_per_block in (8, 16):
+    for rows_per_block in (8, 16, 10, 12, None):
         fused_cache = fresh_cache()
         target = ops.RopeTarget(positions, slots, inv_freq, rot, fused_cache, nq, nkv, d)
         fused_q = ops.gemm_rows(x, w_paired, b_paired, "rope", rope=target, rows_per_block=rows_per_block)
@@ -816,7 +816,7 @@ def test_attention_and_products_at_random_sizes(seed):
     assert rel_err(got, want) < 1e-5, what
     if m <= 16:
         waves = rng.choice([2, 4, 8, 16])
-        rows_per_block = rng.choice([8, 16, 32] if waves <= 8 else [8, 16])
+        rows_per_block = rng.choice([8, 16, 32, 10, 4] if waves <= 8 else [8, 16, 12, 14])
         got = ops.gemm_rows(x.to(DEV), w.to(DEV), b.to(DEV), waves=waves, rows_per_block=rows_per_block).dense()
         assert rel_err(got, want) < 1e-5, (what, waves, rows_per_block)
         if n % 2 == 0:

@@ -50,7 +50,7 @@ struct RowsArgs {
   const uint16_t* w;          // [N, K] bfloat16
   const uint16_t* bias;       // [N] or null
   int M, N, K, k_per_wave;    // k_per_wave: multiple of 64
-  int rows_per_block;         // 16 or 8
+  int rows_per_block;         // even, up to 16; or 32
   // row scale (null: none)
   const float* ssq_in;        // [strips_in, 16] partial sums of squares of the normed input's rows, over any split of its columns
   int strips_in;
@@ -333,7 +333,8 @@ using namespace tlie;
 // 2: residual float [M, N] += y; if xg is given, next_weight [N] (bfloat16 if next_weight_dtype is 1,
 // else float) and xg bfloat16 [M, N]; if ssq_out is given, float [ceil(N / rows_per_block) * max(1, rows_per_block / 16), 16]
 // (all of it is written).
-// waves: 2, 4, 8 or 16, how many waves of a workgroup share K.  rows_per_block: 8, 16, or 32 (32 with at most 8 waves).
+// waves: 2, 4, 8 or 16, how many waves of a workgroup share K.  rows_per_block: an even number up to 16 (the rest of the
+// strip of 16 is idle), or 32 (two strips, with at most 8 waves).
 // 3: the rotation and cache write of rope_cache.hip on W's rows in paired order (see above): positions, slot_map [M],
 // inv_freq [rot_dim / 2] or null, q_out bfloat16 [M, nq * d], cache bfloat16 [pages, 2, nkv, page_size * d];
 // N = (nq + 2 nkv) * d.
@@ -344,7 +345,7 @@ extern "C" int tlie_gemm_rows(const void* x, const void* w, const void* bias, in
                               int nkv, int d, int page_size, void* q_out, void* cache, int waves, int rows_per_block,
                               void* stream) {
   if (M <= 0 || M > 16 || N <= 0 || K <= 0 || (K & 7) != 0 || (waves != 2 && waves != 4 && waves != 8 && waves != 16)) return kBadArgument;
-  if (rows_per_block != 16 && rows_per_block != 8 && !(rows_per_block == 32 && waves <= 8)) return kBadArgument;
+  if (!(rows_per_block >= 2 && rows_per_block <= 16 && rows_per_block % 2 == 0) && !(rows_per_block == 32 && waves <= 8)) return kBadArgument;
   if (ssq_in != nullptr && (strips_in <= 0 || width <= 0)) return kBadArgument;
   if (epilogue == kEpilogueStore && y == nullptr) return kBadArgument;
   if (epilogue == kEpilogueSilu && (act == nullptr || (N & 1) != 0)) return kBadArgument;
