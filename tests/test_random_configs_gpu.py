@@ -1,0 +1,61 @@
+"""Random small configurations and workloads through `Engine.generate`, checked token by token against
+the plain implementation: head sizes that are no power of two, group sizes 1 to 8, widths and
+vocabularies of any size, pages of 4 to 64 rows, pools so small that requests are preempted, token
+budgets and portions of a few tokens.  Every sampled token must be the plain logits' best (32-bit),
+or within the bfloat16 tolerance of the best."""
+import random
+
+import pytest
+import torch
+
+from gpu_helpers import load_plain, make_model
+from plain_llama import plain_forward
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_case(seed):
+    rng = random.Random(seed)
+    dtype = rng.choice(["float32", "bfloat16"])
+    # (bfloat16 takes the matrix-core attention for head sizes that are multiples of 16 and pages of 16
+    # rows or more, and the plain kernel otherwise: both are drawn)
+    head_dim = rng.choice([16, 32, 48, 64, 80, 128, 24]) if dtype == "bfloat16" else rng.choice([8, 12, 16, 24, 32, 40, 64, 100])
+    kv_heads, group = rng.choice([1, 2, 3]), rng.choice([1, 2, 3, 4, 5, 8])
+    heads = kv_heads * group
+    config = dict(model_type="llama", architectures=["LlamaForCausalLM"], hidden_size=rng.choice([64, 96, 72, 128, 200]),
+                  intermediate_size=rng.choice([64, 88, 176, 200, 256, 344]), num_hidden_layers=rng.choice([1, 2, 3]),
+                  num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=head_dim,
+                  max_position_embeddings=rng.choice([96, 160, 300]), vocab_size=rng.choice([50, 127, 256, 1000]),
+                  rms_norm_eps=rng.choice([1e-5, 1e-6]), rope_theta=rng.choice([10000.0, 500000.0]),
+                  tie_word_embeddings=rng.random() < 0.5, attention_bias=rng.random() < 0.4, hidden_act="silu",
+                  bos_token_id=1, eos_token_id=2)
+    page = rng.choice([8, 16, 32, 64]) if dtype == "bfloat16" else rng.choice([4, 8, 16, 32])
+    requests, generated = rng.choice([1, 2, 3, 5, 8, 20]), rng.choice([1, 3, 8, 20, 40])
+    longest = config["max_position_embeddings"] - generated - 1
+    prompts = [[rng.randrange(config["vocab_size"]) for _ in range(rng.randrange(1, max(2, longest)))] for _ in range(requests)]
+    need = max(len(prompt) + generated for prompt in prompts)
+    total = sum(len(prompt) + generated for prompt in prompts)
+    pool = rng.choice([total + page * requests, max(need + page, total // 2), need + page])
+    return dict(dtype=dtype, config=config, page=page, prompts=prompts, generated=generated,
+                pool=(pool + page - 1) // page * page, budget=rng.choice([16, 40, 64, 256, 2048]), chunk=rng.choice([None, 8, 24, 64]))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configuration_and_workload(tmp_path, seed):
+    from tlie_amd import Engine
+    case = draw_case(seed)
+    folder = make_model(tmp_path / "model", case["config"], seed, case["dtype"])
+    raw, weights = load_plain(folder)
+    engine = Engine(folder, dtype=case["dtype"], max_tokens=case["pool"], page_size=case["page"], max_requests=len(case["prompts"]))
+    stats = {}
+    outputs = engine.generate(case["prompts"], max_tokens=case["generated"], max_tokens_per_step=case["budget"],
+                              chunk_size=case["chunk"], stats=stats)
+    engine.cache.check()
+    assert all(free == engine.cache.num_pages for free in engine.cache.free_pages())     # everything was given back
+    tolerance = 2e-5 if case["dtype"] == "float32" else 4e-2
+    for prompt, tokens in zip(case["prompts"], outputs):
+        assert len(tokens) == case["generated"]
+        logits = plain_forward(raw, weights, prompt + tokens)[len(prompt) - 1:len(prompt) + len(tokens) - 1]
+        for index, token in enumerate(tokens):
+            row = logits[index]
+            assert row[token] >= row.max() - tolerance * row.abs().max(), (seed, case["dtype"], len(prompt), index, stats)
