@@ -589,6 +589,17 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   const size_t row = blockIdx.x;                     // token * nq + head
   const float* ml = part_ml + row * nsplit * 2;
   const int lane = threadIdx.x;
+  // Up to 16 parts and a head size up to 64 (a lane, a dim): the lane asks for its parts of O together
+  // with the maxima and sums, so that the kernel waits for memory once, not twice in a row.
+  constexpr int kParts = 16;
+  const bool ahead = nsplit <= kParts && d <= 64;
+  float early[kParts];
+  if (ahead) {
+    const float* column = part_o + row * nsplit * d + min(lane, d - 1);
+#pragma unroll
+    for (int p = 0; p < kParts; ++p)
+      if (p < nsplit) early[p] = column[static_cast<size_t>(p) * d];      // (a branch of the whole wave)
+  }
   float top = -INFINITY;
   for (int p = lane; p < nsplit; p += 64) top = fmaxf(top, ml[p * 2]);
   top = wave_max(top);
@@ -602,6 +613,20 @@ attention_merge_kernel(const float* __restrict__ part_o, const float* __restrict
   total = wave_sum(total);
   __syncthreads();
   const float inv = 1.f / total;
+  if (ahead) {
+    float a = 0.f, b = 0.f;                                // (the same order of additions as below)
+#pragma unroll
+    for (int p = 0; p < kParts; p += 2) {
+      if (p + 1 < nsplit) {
+        a += weight[p] * early[p];
+        b += weight[p + 1] * early[p + 1];
+      } else if (p < nsplit) {
+        a += weight[p] * early[p];
+      }
+    }
+    if (lane < d) out[row * d + lane] = __bfloat16_as_ushort(__float2bfloat16((a + b) * inv));
+    return;
+  }
   for (int i = lane; i < d; i += 64) {
     const float* column = part_o + row * nsplit * d + i;
     float a = 0.f, b = 0.f;
