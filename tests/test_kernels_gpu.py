@@ -770,10 +770,10 @@ def test_rotation_in_paired_order_and_inside_the_product(case):
     paired_q = ops.rope_cache(ops.gemm_skinny(x, w_paired, b_paired), positions, slots, inv_freq, rot, paired_cache, nq, nkv, d,
                               torch.bfloat16, paired=True)
     assert torch.equal(paired_q, plain_q) and torch.equal(paired_cache, plain_cache)
-    for rows_per_block in (8, 16, 10, 12, None):
+    for rows_per_block, waves in ((8, None), (16, None), (10, None), (12, None), (None, None), (32, 4), (32, 8), (32, 2)):
         fused_cache = fresh_cache()
         target = ops.RopeTarget(positions, slots, inv_freq, rot, fused_cache, nq, nkv, d)
-        fused_q = ops.gemm_rows(x, w_paired, b_paired, "rope", rope=target, rows_per_block=rows_per_block)
+        fused_q = ops.gemm_rows(x, w_paired, b_paired, "rope", rope=target, rows_per_block=rows_per_block, waves=waves)
         # the two products sum in another order, so the last bit of a bfloat16 may differ
         assert rel_err(fused_q, plain_q.double()) < 1e-2
         assert rel_err(fused_cache, plain_cache.double()) < 1e-2

@@ -71,3 +71,20 @@ def test_the_skinny_products_launch_shape_is_one_the_kernel_takes():
         split_len, waves, strips = ops.skinny_plan(64, out_features, in_features, 256)
         workgroups = -(-out_features // (16 * waves * strips)) * -(-in_features // split_len)
         assert 128 < workgroups <= 256, (out_features, in_features, split_len, waves, strips)
+
+
+def test_the_few_rows_products_launch_shape_is_one_the_kernel_takes():
+    """Decided on the host from the sizes alone: waves 4, 8 or 16; an even number of rows of W a
+    workgroup up to 16, or 32 with at most 8 waves; the gated product never an odd pairing."""
+    from tlie_amd import ops
+    for rows in (1, 2, 7, 8, 16):
+        for out_features, in_features in ((2560, 2048), (2048, 2048), (11264, 2048), (2048, 5632), (32000, 2048), (6144, 4096),
+                                          (28672, 4096), (4096, 14336), (128256, 4096), (100, 520), (30, 64), (2112, 2048)):
+            for epilogue in ("store", "rope", "silu", "residual"):
+                for units in (256, 304, 64):
+                    waves, rows_per_block = ops.gemm_rows_shape(out_features, in_features, epilogue, units, rows)
+                    assert waves in (4, 8, 16)
+                    assert (rows_per_block % 2 == 0 and 2 <= rows_per_block <= 16) or (rows_per_block == 32 and waves <= 8)
+    assert ops.gemm_rows_shape(2560, 2048, "rope", 256, 8) == (16, 10)          # 256 workgroups, one a compute unit
+    assert ops.gemm_rows_shape(2048, 2048, "residual", 256, 8) == (16, 16)      # a norm's sums follow: strips of 16
+    assert ops.gemm_rows_shape(128256, 4096, "store", 256, 1) == (4, 16) and ops.gemm_rows_shape(128256, 4096, "store", 256, 8) == (4, 32)

@@ -695,7 +695,8 @@ def gemm_rows_takes(rows: int, weight: torch.Tensor, dtype: torch.dtype) -> bool
             and weight.shape[1] % 8 == 0)
 
 
-def gemm_rows_shape(out_features: int, in_features: int, epilogue: str = "store", compute_units: int = 256) -> tuple[int, int]:
+def gemm_rows_shape(out_features: int, in_features: int, epilogue: str = "store", compute_units: int = 256,
+                    rows: int = 1) -> tuple[int, int]:
     """(waves that share K, rows of W per workgroup), measured inside whole decode steps on the
     TinyLlama shapes: about four thousand waves in all, 4 to 16 a workgroup (11264 rows: 4 waves a
     strip of 16, 1.15 ms a step against 1.25 with 8; 2560 rows: 16 waves, against 8 another 0.03 ms
@@ -705,7 +706,11 @@ def gemm_rows_shape(out_features: int, in_features: int, epilogue: str = "store"
     no norm (whose partial sums would grow in number with the workgroups), the rows are shared out
     evenly over the units instead: 2560 rows on 256 workgroups of 10 rather than 160 of 16, 0.7%
     of a step at batch 1 and 8; the same for the output projection (residual and norm sums) measured
-    0.5% slower."""
+    0.5% slower.
+    With 8 rows of x and more, a workgroup's part of x weighs half as much as its 16 rows of W and
+    more (both come through the L2): large matrices then take two strips a workgroup, which halves
+    that share (Llama-3-8B's output head at 8 rows 239 -> 209 us, at 16 rows 269 -> 229; its gate/up
+    61 -> 58, its q/k/v with 8 waves 17.7 -> 16.6; TinyLlama's head at 16 rows 37.6 -> 34.0)."""
     strips = (out_features + 15) // 16
     waves = 4
     while waves < 16 and strips * waves * 2 <= 4096 and in_features >= waves * 2 * 64:
@@ -713,6 +718,8 @@ def gemm_rows_shape(out_features: int, in_features: int, epilogue: str = "store"
     rows_per_block = 8 if (waves == 16 and strips * 16 < 3072 and in_features > 4096) else 16
     if waves == 16 and rows_per_block == 16 and epilogue in ("store", "rope") and compute_units // 2 < strips < compute_units:
         rows_per_block = max(8, (-(-out_features // compute_units) + 1) // 2 * 2)
+    if rows >= 8 and ((waves == 4 and strips * rows >= 14336) or (waves == 8 and in_features >= 4096 and strips >= compute_units)):
+        rows_per_block = 32
     return waves, rows_per_block
 
 
@@ -758,7 +765,7 @@ def gemm_rows(x, weight: torch.Tensor, bias: torch.Tensor | None, epilogue: str 
         if scale.ssq.dim() != 2 or scale.ssq.shape[1] != 16 or scale.ssq.shape[0] == 0:
             raise invalid_shape(f"gemm_rows: ssq {list(scale.ssq.shape)} is not [parts, 16]")
         ssq_in, strips_in, eps = scale.ssq, scale.ssq.shape[0], float(scale.eps)
-    default_waves, default_rows = gemm_rows_shape(out_features, in_features, epilogue, _compute_units(data.device))
+    default_waves, default_rows = gemm_rows_shape(out_features, in_features, epilogue, _compute_units(data.device), rows)
     waves, rows_per_block = waves or default_waves, rows_per_block or default_rows
     if epilogue == "silu" and rows_per_block % 2 != 0:
         raise invalid_argument("gemm_rows: a gate and its up must fall into one block")
