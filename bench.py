@@ -341,6 +341,11 @@ def main() -> int:
                 torch.cuda.empty_cache()
         record["points"] = points
         record["bench_seconds"] = time.perf_counter() - started_all
+    from tlie_amd import ops as kernel_faces
+    # products of many rows that fell from the vendor's library to the plain 32-bit kernel (each many
+    # times slower): a record measured with any would not be this engine's speed
+    record["library_fallbacks"] = kernel_faces.library_fallbacks()
+    assert record["library_fallbacks"] == 0, f"{record['library_fallbacks']} matrix products took the plain kernel instead of the library's"
     print(json.dumps(record))
     return 0
 

@@ -142,14 +142,29 @@ def plain_top_p_distribution(logits: torch.Tensor, temperature: float, top_p: fl
     return out / out.sum()
 
 
+def stored_as(dtype: torch.dtype):
+    """A function that rounds a tensor to `dtype` and widens it again: what storing an
+    activation in that type between two kernels does to it."""
+    return lambda tensor: tensor.to(dtype).double()
+
+
 def plain_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, cfg: dict, trace: dict | None = None,
-                trace_prefix: str = "") -> torch.Tensor:
+                trace_prefix: str = "", stored=None) -> torch.Tensor:
     """One pre-norm block: x + attn(norm(x)), then x + mlp(norm(x)).  src/model.cpp:132-203.
     `trace` receives the five tensors the reference's ModelTrace keeps per layer
-    (src/model.cpp:136-138,176-177,184-185,200-201,204-205)."""
+    (src/model.cpp:136-138,176-177,184-185,200-201,204-205).
+
+    `stored` (default: nothing) is applied to every activation that a 16-bit device path keeps in
+    memory between two operators, as the reference's FP16 path keeps them
+    (src/cuda/model.cu:412-447: normed input, q, k, v, attention output, both projections' results,
+    the gated activation); the residual stays as it is.  With `stored_as(torch.bfloat16)` this is
+    a model of what 16-bit storage alone costs in precision, every sum still being float64: the
+    yardstick for a 16-bit engine's error over many layers, not a second implementation of it."""
     def keep(name, tensor):
         if trace is not None:
             trace[trace_prefix + name] = tensor
+    if stored is None:
+        stored = lambda tensor: tensor
 
     heads = cfg["num_attention_heads"]
     kv_heads = cfg.get("num_key_value_heads", heads)
@@ -160,36 +175,37 @@ def plain_block(x: torch.Tensor, positions: torch.Tensor, w: dict, prefix: str, 
     def bias(name):
         return w.get(prefix + name)
 
-    normed = plain_rms_norm(x, w[prefix + "input_layernorm.weight"], eps)
+    normed = stored(plain_rms_norm(x, w[prefix + "input_layernorm.weight"], eps))
     keep("input_norm", normed)
-    q = plain_linear(normed, w[prefix + "self_attn.q_proj.weight"], bias("self_attn.q_proj.bias"))
-    k = plain_linear(normed, w[prefix + "self_attn.k_proj.weight"], bias("self_attn.k_proj.bias"))
-    v = plain_linear(normed, w[prefix + "self_attn.v_proj.weight"], bias("self_attn.v_proj.bias"))
-    q = plain_rope(q.view(tokens, heads, head_dim), positions, theta)
-    k = plain_rope(k.view(tokens, kv_heads, head_dim), positions, theta)
-    attended = plain_attention(q, k, v.view(tokens, kv_heads, head_dim))
-    projected = plain_linear(attended.reshape(tokens, heads * head_dim),
-                             w[prefix + "self_attn.o_proj.weight"], bias("self_attn.o_proj.bias"))
+    q = stored(plain_linear(normed, w[prefix + "self_attn.q_proj.weight"], bias("self_attn.q_proj.bias")))
+    k = stored(plain_linear(normed, w[prefix + "self_attn.k_proj.weight"], bias("self_attn.k_proj.bias")))
+    v = stored(plain_linear(normed, w[prefix + "self_attn.v_proj.weight"], bias("self_attn.v_proj.bias")))
+    q = stored(plain_rope(q.view(tokens, heads, head_dim), positions, theta))
+    k = stored(plain_rope(k.view(tokens, kv_heads, head_dim), positions, theta))
+    attended = stored(plain_attention(q, k, v.view(tokens, kv_heads, head_dim)))
+    projected = stored(plain_linear(attended.reshape(tokens, heads * head_dim),
+                                    w[prefix + "self_attn.o_proj.weight"], bias("self_attn.o_proj.bias")))
     keep("attention_output", projected)
     x = x + projected
-    normed = plain_rms_norm(x, w[prefix + "post_attention_layernorm.weight"], eps)
+    normed = stored(plain_rms_norm(x, w[prefix + "post_attention_layernorm.weight"], eps))
     keep("post_attention_norm", normed)
-    gate = plain_linear(normed, w[prefix + "mlp.gate_proj.weight"])
-    up = plain_linear(normed, w[prefix + "mlp.up_proj.weight"])
-    projected = plain_linear(plain_silu_mul(gate, up), w[prefix + "mlp.down_proj.weight"])
+    gate = stored(plain_linear(normed, w[prefix + "mlp.gate_proj.weight"]))
+    up = stored(plain_linear(normed, w[prefix + "mlp.up_proj.weight"]))
+    projected = stored(plain_linear(stored(plain_silu_mul(gate, up)), w[prefix + "mlp.down_proj.weight"]))
     keep("mlp_output", projected)
     keep("output", x + projected)
     return x + projected
 
 
-def plain_forward(cfg: dict, w: dict, tokens: list[int], first_position: int = 0, trace: dict | None = None) -> torch.Tensor:
+def plain_forward(cfg: dict, w: dict, tokens: list[int], first_position: int = 0, trace: dict | None = None,
+                  stored=None) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.  src/model.cpp:80-234.
 
     Embedding row copy (:94-97), the blocks in order (:112-207), final norm (:217) and the
     output projection (:224-225); with tied embeddings the output projection is the
     embedding table.  `first_position` shifts every position; it is for the tests' invariants.
     `trace` receives the named tensors of the reference's ModelTrace ("embedding", "layerN.*",
-    "final_norm", "logits": src/model.cpp:98-99,221-222,229-230).
+    "final_norm", "logits": src/model.cpp:98-99,221-222,229-230).  `stored`: see `plain_block`.
     """
     ids = torch.tensor(tokens, dtype=torch.long)
     positions = torch.arange(len(tokens)) + first_position
@@ -197,8 +213,10 @@ def plain_forward(cfg: dict, w: dict, tokens: list[int], first_position: int = 0
     if trace is not None:
         trace["embedding"] = x
     for layer in range(cfg["num_hidden_layers"]):
-        x = plain_block(x, positions, w, f"model.layers.{layer}.", cfg, trace, f"layer{layer}.")
+        x = plain_block(x, positions, w, f"model.layers.{layer}.", cfg, trace, f"layer{layer}.", stored)
     normed = plain_rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
+    if stored is not None:
+        normed = stored(normed)
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     logits = plain_linear(normed, head)
     if trace is not None:

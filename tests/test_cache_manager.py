@@ -10,7 +10,7 @@ import torch
 
 from tlie_amd import EngineError, ErrorCode
 from tlie_amd.cache import ABSENT, CacheManager, PageAllocator, RunNeed
-from tlie_amd.parts import KVCacheNeed, StateNeed
+from tlie_amd.parts import CacheNeed, StateNeed
 
 
 def test_allocator_fifo_all_or_nothing_and_double_free():
@@ -32,7 +32,7 @@ def test_allocator_fifo_all_or_nothing_and_double_free():
 
 
 def manager(num_pages=8, page_size=4, max_requests=3, window=None, state=False, runs=2):
-    needs = [RunNeed(cache_of=i, kv=KVCacheNeed(2, 8, window), state=StateNeed((5,)) if state else None) for i in range(runs)]
+    needs = [RunNeed(cache_of=i, cache=CacheNeed((2, 2), 8, window), state=StateNeed((5,)) if state else None) for i in range(runs)]
     return CacheManager(needs, page_size, num_pages, max_requests, torch.float32, "cpu", max_positions=64)
 
 
@@ -136,16 +136,36 @@ def test_request_slots_run_out_and_state_starts_at_zero():
     assert cache.bindings[0].state is not cache.bindings[1].state
 
 
+def test_pages_of_other_shapes_and_types():
+    """What a page looks like is the mixer's need, not the manager's: one vector per position in
+    a type of its own, three planes, or attention's two planes per head, side by side; runs with
+    the same window share page numbers whatever their pages hold."""
+    needs = [RunNeed(0, CacheNeed((), 24, None, torch.float16)), RunNeed(1, CacheNeed((3,), 5, None)),
+             RunNeed(2, CacheNeed((2, 2), 8, None)), RunNeed(0, CacheNeed((), 24, None, torch.float16))]
+    cache = CacheManager(needs, 4, 6, 2, torch.float32, "cpu")
+    assert len(cache.groups) == 1 and [b.group for b in cache.bindings] == [0, 0, 0, 0]
+    assert cache.bindings[0].cache.shape == (6, 4 * 24) and cache.bindings[0].cache.dtype == torch.float16
+    assert cache.bindings[1].cache.shape == (6, 3, 4 * 5) and cache.bindings[1].cache.dtype == torch.float32
+    assert cache.bindings[2].cache.shape == (6, 2, 2, 4 * 8)
+    assert cache.bindings[3].cache is cache.bindings[0].cache and not cache.bindings[3].writes
+    assert CacheManager.page_bytes(needs, 4, torch.float32) == 4 * (24 * 2 + 15 * 4 + 32 * 4)
+    assert CacheNeed((2, 3), 7).page_shape(16) == (2, 3, 112) and CacheNeed((), 9).values_per_position() == 9
+    with pytest.raises(EngineError):         # a reader whose pages are of another type than the owner's
+        CacheManager([RunNeed(0, CacheNeed((), 24, None, torch.float16)), RunNeed(0, CacheNeed((), 24))], 4, 6, 2, torch.float32, "cpu")
+    with pytest.raises(EngineError):         # a budget counts each pool in its own type
+        CacheManager(needs, 4, 6, 2, torch.float32, "cpu", max_bytes=6 * 4 * (24 * 2 + 15 * 4 + 32 * 4) - 1)
+
+
 def test_groups_by_need_and_shared_caches():
-    needs = [RunNeed(0, KVCacheNeed(2, 8, None)), RunNeed(1, KVCacheNeed(1, 16, 6)), RunNeed(0, KVCacheNeed(2, 8, None)),
-             RunNeed(3, None), RunNeed(4, KVCacheNeed(2, 8, 6))]
+    needs = [RunNeed(0, CacheNeed((2, 2), 8, None)), RunNeed(1, CacheNeed((2, 1), 16, 6)), RunNeed(0, CacheNeed((2, 2), 8, None)),
+             RunNeed(3, None), RunNeed(4, CacheNeed((2, 2), 8, 6))]
     cache = CacheManager(needs, 4, 6, 2, torch.float32, "cpu")
     assert [group.window for group in cache.groups] == [None, 6]
     assert [b.group for b in cache.bindings] == [0, 1, 0, None, 1]
     assert cache.bindings[2].cache is cache.bindings[0].cache and not cache.bindings[2].writes and cache.bindings[0].writes
     assert cache.bindings[1].cache.shape == (6, 2, 1, 4 * 16) and cache.bindings[4].cache.shape == (6, 2, 2, 4 * 8)
     with pytest.raises(EngineError):
-        CacheManager([RunNeed(0, KVCacheNeed(2, 8)), RunNeed(0, KVCacheNeed(1, 8))], 4, 6, 2, torch.float32, "cpu")
+        CacheManager([RunNeed(0, CacheNeed((2, 2), 8)), RunNeed(0, CacheNeed((2, 1), 8))], 4, 6, 2, torch.float32, "cpu")
     # the windowed group gives pages back as the request grows; the full group keeps them
     cache.admit("a")
     for _ in range(5):
@@ -221,7 +241,7 @@ def test_random_orders_lose_nothing(seed):
 
 def test_a_byte_budget_refuses_a_pool_before_it_is_allocated():
     """src/kv_cache.cpp:40-43: more than the configured bytes is out_of_memory."""
-    needs = [RunNeed(0, KVCacheNeed(2, 8)), RunNeed(1, KVCacheNeed(2, 8)), RunNeed(0, KVCacheNeed(2, 8))]   # two pools, one reader
+    needs = [RunNeed(0, CacheNeed((2, 2), 8)), RunNeed(1, CacheNeed((2, 2), 8)), RunNeed(0, CacheNeed((2, 2), 8))]   # two pools, one reader
     per_page = CacheManager.page_bytes(needs, 4, torch.float32)
     assert per_page == 2 * (2 * 2 * 4 * 8 * 4)
     CacheManager(needs, 4, 10, 2, torch.float32, "cpu", max_bytes=10 * per_page)

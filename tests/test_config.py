@@ -100,6 +100,28 @@ def test_spec_is_data():
         replace(spec, runs=(Run(0, 0), Run(1, 0), Run(1, 1))).validate()   # run 2 reads run 1, which owns none
 
 
+def test_a_head_size_the_kernels_do_not_take_is_refused_where_the_part_is_built():
+    """Not by the first step's launch: building the attention part (as the engine does when it
+    builds the model) refuses a head size beyond the kernels', with the limit in the message."""
+    import torch
+    from tlie_amd.config import PartSpec
+    from tlie_amd.parts.attention import Attention
+
+    def build(head_dim, heads=2, kv_heads=1):
+        position = PartSpec("rotary", {"head_dim": head_dim, "theta": 1e4})
+        return Attention(PartSpec("attention", {"hidden_size": 64, "num_heads": heads, "num_kv_heads": kv_heads, "head_dim": head_dim,
+                                                "position": position}), torch.bfloat16, "cpu")
+    assert build(256).d == 256
+    with pytest.raises(EngineError) as caught:
+        build(272)
+    assert caught.value.code == ErrorCode.INVALID_CONFIG and "272" in caught.value.message and "256" in caught.value.message
+    assert code_of(lambda: build(64, heads=3, kv_heads=2)) == ErrorCode.INVALID_CONFIG
+    # the model built from a configuration goes the same way
+    from tlie_amd.models.builder import DecoderModel
+    wide = config_from_dict(dict(FIXTURE, head_dim=320, num_hidden_layers=1))
+    assert code_of(lambda: DecoderModel(wide.to_spec(), torch.bfloat16, "cpu")) == ErrorCode.INVALID_CONFIG
+
+
 def test_error_json_shape():
     error = tlie_amd.EngineError(ErrorCode.OUT_OF_BOUNDS, "x")
     assert json.loads(error.to_json()) == {"error": {"code": "out_of_bounds", "message": "x"}}

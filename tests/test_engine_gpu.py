@@ -111,10 +111,12 @@ def test_named_intermediate_tensors_layer_by_layer(setups, name, dtype):
 @pytest.mark.parametrize("name", sorted(CONFIGS))
 def test_named_intermediate_tensors_on_the_route_of_few_rows(setups, name):
     """A bfloat16 step of at most 16 tokens (what decoding runs) folds the norms into its products
-    and lets the products add into the residual themselves; with a trace it takes that same route
-    and leaves what still exists there as a tensor: per layer what the mixer and the feed-forward
-    added and the layer's output, the embedding and the logits.  Steps of 9, 5, 1 and 1 tokens after
-    a prompt portion, each name against the plain implementation's rows at those positions."""
+    and lets the products add into the residual themselves; a trace that asks for the serving route
+    takes that same route and leaves what still exists there as a tensor: per layer what the mixer and
+    the feed-forward added and the layer's output, the embedding and the logits.  Steps of 9, 5, 1 and
+    1 tokens after a prompt portion, each name against the plain implementation's rows at those
+    positions.  Without that request the same steps leave every name of the reference's trace, and the
+    two routes' logits agree within the tolerance of two cuts."""
     setup = setups(name, "bfloat16")
     engine = new_engine(setup, "bfloat16")
     tokens = request_tokens(name, 4, 45)
@@ -127,9 +129,24 @@ def test_named_intermediate_tensors_on_the_route_of_few_rows(setups, name):
     start, traces = 29, []
     for count in (9, 5, 1, 1):
         traces.append({})
-        engine.step([StepEntry("t", tokens[start:start + count], list(range(count)))], trace=traces[-1])
+        engine.step([StepEntry("t", tokens[start:start + count], list(range(count)))], trace=traces[-1], trace_serving_route=True)
         start += count
     engine.finish("t")
+    # by default a traced step of few rows leaves all the names, like any other step
+    engine.admit("f")
+    engine.step([StepEntry("f", tokens[:29], [])])
+    full, start = [], 29
+    for count in (9, 5, 1, 1):
+        full.append({})
+        engine.step([StepEntry("f", tokens[start:start + count], list(range(count)))], trace=full[-1])
+        start += count
+    engine.finish("f")
+    for trace in full:
+        assert sorted(trace) == sorted(plain)
+    for key in plain:
+        assert_close(torch.cat([trace[key] for trace in full]).cpu(), plain[key][29:], TOLERANCE["bfloat16"], "every name: " + key)
+    assert_close(torch.cat([trace["logits"] for trace in full]).cpu(), torch.cat([trace["logits"] for trace in traces]).cpu().double(),
+                 CUT_TOLERANCE["bfloat16"], "the two routes' logits")
     names = ["embedding"] + [f"layer{layer}.{part}" for layer in range(layers) for part in ("attention_output", "mlp_output", "output")] \
         + ["logits"]
     for trace in traces:

@@ -269,6 +269,12 @@ def test_attention_that_shares_keys_among_neighbouring_tokens_gives_the_same_bit
     shared = ops.attention_generic(*arguments, tiled=True)
     assert torch.isfinite(shared.float()).all()
     assert torch.equal(alone, shared)
+    # a mixed step launches both forms, and each sequence's token count decides which one serves it: the
+    # single token goes to the first form (and, with a higher bar, the portion of 89 tokens too)
+    seq_start = torch.tensor([0, 613, 614, 703], dtype=torch.int32, device=DEV)
+    for bar in (4, 100, 1000):
+        split = ops.attention_generic(*arguments, tiled=2, seq_start=seq_start, min_tokens=bar)
+        assert torch.equal(alone, split), f"served by both forms, sequences of {bar} tokens and more by the second"
     assert rel_err(shared.view(-1, nq, d)[:-padding], torch.cat(wants)) < TOL[dtype]
 
 

@@ -395,6 +395,279 @@ def test_toy_parts_register_build_and_step(tmp_path):
     assert engine.cache.free_slots == 3
 
 
+def register_recorded_state_toy():
+    """A mixer with state of its own that may be recorded: every operation is a launch on the
+    current stream whose sizes depend on the token and sequence counts alone.  It reads the
+    request slots from the device (`token_slot`, `seq_slot`) and moves the state of live rows
+    only: a recorded step's padding has slot -1."""
+    from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run, TensorSpec
+    from tlie_amd.parts import Mixer, StateNeed
+    from tlie_amd.parts.linear import Linear
+    from tlie_amd.registry import register
+
+    @register("mixer", "toy_recorded_running_mean")
+    class RecordedRunningMean(Mixer):
+        """out[t] = W . mean(x[0..t]) with the running sum as the request's state."""
+        graph_safe = True
+
+        @classmethod
+        def tensor_specs(cls, spec, prefix):
+            return [TensorSpec(prefix + "mix.weight", (spec["hidden_size"], spec["hidden_size"]))]
+
+        def load(self, weights, prefix):
+            self.mix = Linear(weights[prefix + "mix.weight"], None, self.dtype)
+
+        def state_need(self):
+            return StateNeed((self.spec["hidden_size"],), torch.float32)
+
+        def forward(self, x, ctx, binding):
+            count = x.shape[0]
+            live = ctx.token_slot >= 0
+            rows = ctx.token_slot.long().clamp(min=0)
+            values = x.float() * live[:, None]                       # padding tokens count for nothing
+            index = torch.arange(count, device=x.device)
+            before = (ctx.token_seq[:, None] == ctx.token_seq[None, :]) & (index[None, :] <= index[:, None]) & live[None, :]
+            sums = (before[:, :, None] * values[None, :, :]).sum(dim=1) + binding.state[rows]
+            # the state moves for sequences that ran, once each; a padding sequence adds zeros
+            sequence = torch.arange(ctx.num_seqs, device=x.device)
+            member = (ctx.token_seq[None, :] == sequence[:, None]) & live[None, :]
+            totals = (member[:, :, None] * values[None, :, :]).sum(dim=1) * (ctx.seq_slot >= 0)[:, None]
+            binding.state.index_add_(0, ctx.seq_slot.long().clamp(min=0), totals)
+            means = sums / (ctx.positions.float() + 1.0)[:, None]
+            return self.mix(means.to(self.dtype).contiguous())
+
+    @register("architecture", "ToyRecordedStateForCausalLM")
+    @dataclass(frozen=True)
+    class RecordedStateConfig:
+        hidden_size: int
+        vocab_size: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["hidden_size"], raw["vocab_size"], raw["eps"])
+
+        def to_dict(self):
+            return {"architectures": ["ToyRecordedStateForCausalLM"], "hidden_size": self.hidden_size,
+                    "vocab_size": self.vocab_size, "eps": self.eps}
+
+        def to_spec(self):
+            norm = PartSpec("rms_norm", {"size": self.hidden_size, "eps": self.eps})
+            attention = PartSpec("attention", {"hidden_size": self.hidden_size, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                               "bias": False, "window": None,
+                                               "position": PartSpec("rotary", {"head_dim": 16, "theta": 100.0})})
+            mean = PartSpec("toy_recorded_running_mean", {"hidden_size": self.hidden_size})
+            mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 40, "activation": "silu"})
+            layers = (LayerSpec("model.layers.0.", "pre_norm", attention, mlp, norm, norm),
+                      LayerSpec("model.layers.1.", "pre_norm", mean, mlp, norm, norm))
+            return ModelSpec("ToyRecordedStateForCausalLM", self.hidden_size, self.vocab_size, 128,
+                             PartSpec("token_embedding", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size}),
+                             layers, (Run(0, 0), Run(1, 1)), norm,
+                             PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "tied": False}))
+    return RecordedStateConfig
+
+
+def plain_recorded_state_forward(raw, w, tokens):
+    count, eps = len(tokens), raw["eps"]
+    x = w["model.embed_tokens.weight"][tokens]
+
+    def mlp(x, p):
+        normed = plain_rms_norm(x, w[p + "post_attention_layernorm.weight"], eps)
+        return plain_linear(plain_silu_mul(plain_linear(normed, w[p + "mlp.gate_proj.weight"]),
+                                           plain_linear(normed, w[p + "mlp.up_proj.weight"])), w[p + "mlp.down_proj.weight"])
+    p = "model.layers.0."
+    x = x + plain_attention_part(plain_rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", 2, 1, 16, 100.0, None, False)
+    x = x + mlp(x, p)
+    p = "model.layers.1."
+    normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)
+    means = torch.cumsum(normed, dim=0) / (torch.arange(count).double() + 1.0)[:, None]
+    x = x + plain_linear(means, w[p + "self_attn.mix.weight"])
+    x = x + mlp(x, p)
+    return plain_linear(plain_rms_norm(x, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_state_of_fixed_size_in_recorded_steps(tmp_path, dtype):
+    """A request's state row moves only for rows that ran (reference: `next_positions` moves for
+    the step's own slots only, src/cuda/model.cu:550-554,721-723).  A recorded step pads its
+    sequences and tokens; the request in slot 0 runs beside that padding, in recorded steps of
+    portions and of single tokens, several replays each, and its logits stay the plain ones:
+    they would not if padding rows carried slot 0, as any live row may."""
+    from tlie_amd import Engine, write_random_model
+    from gpu_helpers import Replayer
+    config = register_recorded_state_toy()(hidden_size=32, vocab_size=80, eps=1e-5)
+    write_random_model(str(tmp_path), config, seed=21, std=0.15, norm_std=0.1,
+                       dtype=torch.float32 if dtype == "float32" else torch.bfloat16)
+    raw, weights = load_plain(str(tmp_path))
+    tolerance = 2e-5 if dtype == "float32" else 3e-2
+    engine = Engine(str(tmp_path), dtype=dtype, max_tokens=512, page_size=16, max_requests=4)
+    assert engine.runner.use_graphs and engine.cache.bindings[1].state.shape == (4, 32)
+    streams = {"a": [(7 * i * i + 3) % 80 for i in range(60)], "b": [(5 * i + 1) % 80 for i in range(45)],
+               "c": [(11 * i + 2 * (i % 3)) % 80 for i in range(33)]}
+    want = {request: plain_recorded_state_forward(raw, weights, tokens) for request, tokens in streams.items()}
+    replay = Replayer(engine)
+    engine.admit("a")
+    assert engine.cache.slot("a") == 0
+    # portions: 5 + 3 tokens in a recording of 16 tokens and 8 sequences, replayed with other cuts
+    replay.step([("a", streams["a"][:5], [4]), ("b", streams["b"][:3], [2])])
+    replay.step([("a", streams["a"][5:12], [6]), ("b", streams["b"][3:9], [5])])
+    replay.step([("b", streams["b"][9:20], [10]), ("c", streams["c"][:2], [1]), ("a", streams["a"][12:13], [0])])
+    recording = next(iter(engine.runner._portion_graphs.values()))
+    assert recording.graph is not None, "the steps of portions were not replayed from a recording"
+    assert (recording.host["seq_slot"][3:] == -1).all() and (recording.host["token_slot"][14:] == -1).all()
+    assert sorted(recording.host["seq_slot"][:3].tolist()) == [0, 1, 2]
+    done = {"a": 13, "b": 20, "c": 2}
+    # single tokens: three requests in a recording of four rows (one row of padding), many replays
+    for _ in range(12):
+        replay.step([(request, streams[request][done[request]:done[request] + 1], [0]) for request in ("c", "a", "b")])
+        for request in done:
+            done[request] += 1
+    decode = next(iter(engine.runner._graphs.values()))
+    assert decode.bucket == 4 and decode.graph is not None and decode.host["seq_slot"][3] == -1 and decode.host["token_slot"][3] == -1
+    # "c" ends; its slot and state row are taken by "d", which starts from zero beside the others
+    engine.finish("c")
+    streams["d"], want["d"] = streams["c"], want["c"]
+    done["d"] = 0
+    replay.step([("a", streams["a"][done["a"]:done["a"] + 1], [0]), ("d", streams["d"][:9], [8])])
+    done["a"], done["d"] = done["a"] + 1, 9
+    for _ in range(10):
+        replay.step([(request, streams[request][done[request]:done[request] + 1], [0]) for request in ("a", "b", "d")])
+        for request in ("a", "b", "d"):
+            done[request] += 1
+    keys = sorted(replay.rows, key=str)
+    for request in ("a", "b", "c", "d"):
+        places = [place for name, place in keys if name == request]
+        assert len(places) >= 11
+        assert_close(replay.logits_of(request, places), want[request][places], tolerance, f"request {request}")
+    # the state rows hold the running sums of exactly the tokens that ran
+    for request in ("a", "b", "d"):
+        engine.finish(request)
+    assert engine.cache.free_slots == 4
+
+
+def register_latent_cache_toy():
+    """A mixer that keeps one vector per position in pages of its own shape and type, and an
+    architecture that runs it beside an attention layer: the two runs share page numbers (one
+    group), their pools have nothing else in common."""
+    from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run, TensorSpec
+    from tlie_amd.parts import CacheNeed, Mixer
+    from tlie_amd.parts.linear import Linear
+    from tlie_amd.registry import register
+
+    @register("mixer", "toy_latent_mean")
+    class LatentMean(Mixer):
+        """Caches latent[t] = P . x[t] (float32, `latent` values per position, one plane) and
+        gives out[t] = W . mean(latent[0..t]), read back from the pages through the block table."""
+
+        @classmethod
+        def tensor_specs(cls, spec, prefix):
+            return [TensorSpec(prefix + "down.weight", (spec["latent"], spec["hidden_size"])),
+                    TensorSpec(prefix + "up.weight", (spec["hidden_size"], spec["latent"]))]
+
+        def load(self, weights, prefix):
+            self.down = Linear(weights[prefix + "down.weight"], None, self.dtype)
+            self.up = Linear(weights[prefix + "up.weight"], None, self.dtype)
+
+        def cache_need(self):
+            return CacheNeed((), int(self.spec["latent"]), None, torch.float32)
+
+        def forward(self, x, ctx, binding):
+            width = int(self.spec["latent"])
+            latent = ops.as_product(self.down(x, out_dtype=torch.float32)).dense(torch.float32)
+            rows = binding.cache.view(-1, width)                       # [pages * page_size, latent]
+            page_size = binding.cache.shape[1] // width
+            group = binding.group
+            rows[ctx.groups[group].slot_map.long()] = latent
+            table, starts = ctx.host[f"block_table{group}"], ctx.host["seq_start"]
+            means = torch.empty_like(latent)
+            for index in range(ctx.num_seqs):
+                begin, end, length = int(starts[index]), int(starts[index + 1]), int(ctx.host["seq_len"][index])
+                where = torch.tensor([int(table[index, p // page_size]) * page_size + p % page_size for p in range(length)],
+                                     device=x.device)
+                running = torch.cumsum(rows[where], dim=0) / torch.arange(1, length + 1, device=x.device)[:, None]
+                means[begin:end] = running[length - (end - begin):]
+            return self.up(means.to(self.dtype).contiguous())
+
+    @register("architecture", "ToyLatentForCausalLM")
+    @dataclass(frozen=True)
+    class LatentConfig:
+        hidden_size: int
+        vocab_size: int
+        latent: int
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["hidden_size"], raw["vocab_size"], raw["latent"])
+
+        def to_dict(self):
+            return {"architectures": ["ToyLatentForCausalLM"], "hidden_size": self.hidden_size, "vocab_size": self.vocab_size,
+                    "latent": self.latent}
+
+        def to_spec(self):
+            norm = PartSpec("rms_norm", {"size": self.hidden_size, "eps": 1e-5})
+            attention = PartSpec("attention", {"hidden_size": self.hidden_size, "num_heads": 2, "num_kv_heads": 2, "head_dim": 16,
+                                               "bias": False, "window": None,
+                                               "position": PartSpec("rotary", {"head_dim": 16, "theta": 50.0})})
+            latent = PartSpec("toy_latent_mean", {"hidden_size": self.hidden_size, "latent": self.latent})
+            mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 48, "activation": "silu"})
+            layers = (LayerSpec("model.layers.0.", "pre_norm", latent, mlp, norm, norm),
+                      LayerSpec("model.layers.1.", "pre_norm", attention, mlp, norm, norm))
+            return ModelSpec("ToyLatentForCausalLM", self.hidden_size, self.vocab_size, 128,
+                             PartSpec("token_embedding", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size}),
+                             layers, (Run(0, 0), Run(1, 1)), norm,
+                             PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "tied": False}))
+    return LatentConfig
+
+
+def test_a_mixer_whose_pages_hold_one_vector_per_position(tmp_path):
+    """The cache manager allocates what a mixer's need says and knows nothing of keys or values:
+    a toy mixer with pages [page_size * latent] of float32 beside an attention layer's
+    [2, heads, page_size * d], on the same page numbers; whole, in portions beside another request,
+    and with pages that an ended request gave back."""
+    from tlie_amd import Engine, write_random_model
+    from gpu_helpers import Replayer
+    config = register_latent_cache_toy()(hidden_size=32, vocab_size=70, latent=5)
+    write_random_model(str(tmp_path), config, seed=4, std=0.15, norm_std=0.1, dtype=torch.float32)
+    raw, w = load_plain(str(tmp_path))
+
+    def plain(tokens):
+        count = len(tokens)
+        x = w["model.embed_tokens.weight"][tokens]
+
+        def mlp(x, p):
+            normed = plain_rms_norm(x, w[p + "post_attention_layernorm.weight"], 1e-5)
+            return plain_linear(plain_silu_mul(plain_linear(normed, w[p + "mlp.gate_proj.weight"]),
+                                               plain_linear(normed, w[p + "mlp.up_proj.weight"])), w[p + "mlp.down_proj.weight"])
+        p = "model.layers.0."
+        latent = plain_linear(plain_rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), w[p + "self_attn.down.weight"])
+        means = torch.cumsum(latent, dim=0) / (torch.arange(count).double() + 1.0)[:, None]
+        x = x + plain_linear(means, w[p + "self_attn.up.weight"])
+        x = x + mlp(x, p)
+        p = "model.layers.1."
+        x = x + plain_attention_part(plain_rms_norm(x, w[p + "input_layernorm.weight"], 1e-5), w, p + "self_attn.", 2, 2, 16, 50.0, None, False)
+        x = x + mlp(x, p)
+        return plain_linear(plain_rms_norm(x, w["model.norm.weight"], 1e-5), w["lm_head.weight"])
+
+    engine = Engine(str(tmp_path), dtype="float32", max_tokens=96, page_size=8, max_requests=3)
+    assert len(engine.cache.groups) == 1
+    assert engine.cache.bindings[0].cache.shape == (12, 8 * 5) and engine.cache.bindings[0].cache.dtype == torch.float32
+    assert engine.cache.bindings[1].cache.shape == (12, 2, 2, 8 * 16)
+    tokens = [(13 * i * i + 5) % 70 for i in range(50)]
+    other = [(3 * i + 1) % 70 for i in range(30)]
+    want, want_other = plain(tokens), plain(other)
+    replay = Replayer(engine)
+    replay.step([("whole", tokens, list(range(50)))], end=["whole"])
+    assert_close(replay.logits_of("whole", range(50)), want, 2e-5, "whole")
+    replay.step([("a", tokens[:11], list(range(11))), ("b", other, list(range(30)))], end=["b"])
+    replay.step([("a", tokens[11:13], [0, 1]), ("c", other[:17], list(range(17)))])       # "c" on pages that "b" gave back
+    replay.step([("c", other[17:], list(range(13))), ("a", tokens[13:14], [0])], end=["c"])
+    replay.step([("a", tokens[14:], list(range(36)))], end=["a"])
+    assert_close(replay.logits_of("a", range(50)), want, 2e-5, "in portions")
+    assert_close(replay.logits_of("b", range(30)), want_other, 2e-5, "beside it")
+    assert_close(replay.logits_of("c", range(30)), want_other, 2e-5, "on pages that were used before")
+    assert engine.cache.free_pages() == [12]
+
+
 def register_windowed_toy():
     """A second architecture of the test's own, out of the framework's parts only: a layer whose
     attention sees a window of 11 positions (its pages come back while a request runs) and turns

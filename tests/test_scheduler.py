@@ -7,11 +7,11 @@ import torch
 from tlie_amd import EngineError, ErrorCode
 from tlie_amd.cache import CacheManager, RunNeed
 from tlie_amd.engine import Request, SamplingParams, Scheduler
-from tlie_amd.parts import KVCacheNeed
+from tlie_amd.parts import CacheNeed
 
 
 def make(num_pages=16, page_size=4, max_requests=4, **kwargs):
-    cache = CacheManager([RunNeed(0, KVCacheNeed(1, 8))], page_size, num_pages, max_requests, torch.float32, "cpu",
+    cache = CacheManager([RunNeed(0, CacheNeed((2, 1), 8))], page_size, num_pages, max_requests, torch.float32, "cpu",
                          max_positions=kwargs.pop("max_positions", 64))
     return cache, Scheduler(cache, max_positions=cache.max_positions, **kwargs)
 

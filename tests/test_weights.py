@@ -78,12 +78,16 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     tensors["model.layers.0.extra.weight"] = torch.zeros(2).bfloat16()
     tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(4)         # a stored buffer: ignored
     write_safetensors(str(tmp_path / "model.safetensors"), tensors)
-    error = code_of(lambda: WeightStore(str(tmp_path)).load(specs, torch.bfloat16, "cpu"))
+    ignored = config.to_spec().ignored_tensors
+    error = code_of(lambda: WeightStore(str(tmp_path)).load(specs, torch.bfloat16, "cpu", ignored))
     assert error.code == ErrorCode.INVALID_SHAPE
     for piece in ("2 missing", "model.layers.1.mlp.up_proj.weight", "model.norm.weight", "1 unexpected",
                   "model.layers.0.extra.weight", "1 with a wrong shape", "stored [32, 31], expected [32, 32]"):
         assert piece in error.message, piece
     assert "inv_freq" not in error.message
+    # which names may be carried unread is the architecture's: the store itself knows none
+    error = code_of(lambda: WeightStore(str(tmp_path)).load(specs, torch.bfloat16, "cpu"))
+    assert "2 unexpected" in error.message and "rotary_emb.inv_freq" in error.message
 
 
 def test_tied_model_may_carry_its_head(tmp_path):

@@ -2,7 +2,8 @@
 it (through ctypes): paged attention with the partial results of its key parts in the library's own
 device array instead of buffers of the caller's.  Its output is compared, bit for bit, with that of
 the entry point that takes buffers, on two calls in a row, the second smaller than the first (the
-array still holds the first call's contents); and a step beyond the array's size is refused."""
+array still holds the first call's contents), and with the plain attention on the same keys and
+values read back out of the pages; and a step beyond the array's size is refused."""
 import ctypes
 
 import pytest
@@ -22,6 +23,29 @@ def make_case(seed, seqs, length, nq, nkv, d, page_size=16):
     q = (torch.randn((seqs, nq * d), generator=generator)).to(torch.bfloat16).cuda()
     positions = torch.full((seqs,), length - 1, dtype=torch.int32).cuda()
     return q, cache, table, positions
+
+
+def plain_decode_attention(q, cache, table, length, nq, nkv, d, page_size=16):
+    """The plain attention's answer for the last position of every sequence: keys and values are
+    gathered out of the pages (keys [row][dim], values [dim][row]) into whole sequences first."""
+    rows = []
+    for seq in range(q.shape[0]):
+        pages = cache[table[seq].long()].double().cpu()                                   # [blocks, 2, nkv, page_size * d]
+        keys = pages[:, 0].reshape(-1, nkv, page_size, d).permute(0, 2, 1, 3).reshape(-1, nkv, d)[:length]
+        values = pages[:, 1].reshape(-1, nkv, d, page_size).permute(0, 3, 1, 2).reshape(-1, nkv, d)[:length]
+        rows.append(last_row_attention(q[seq].double().cpu().view(nq, d), keys, values, nq // nkv))
+    return torch.stack(rows).reshape(q.shape[0], nq * d)
+
+
+def last_row_attention(query, keys, values, groups):
+    """softmax(q . K^T / sqrt(d)) . V for one query per head over all `keys` (src/operators.cpp:117-143)."""
+    from plain_llama import plain_softmax
+    d = query.shape[-1]
+    out = torch.zeros_like(query)
+    for head in range(query.shape[0]):
+        scores = (keys[:, head // groups] @ query[head]) * (1.0 / d ** 0.5)
+        out[head] = plain_softmax(scores) @ values[:, head // groups]
+    return out
 
 
 def call_no_alloc(library, q, cache, table, positions, nq, nkv, d, page_size, scale, nsplit, split_len, waves):
@@ -53,6 +77,9 @@ def test_attention_without_allocation_equals_the_entry_point_that_takes_buffers(
         assert status == 0
         assert torch.equal(got, want), f"{seqs} sequences of {length}: the output differs from the entry point with buffers"
         assert torch.isfinite(got.float()).all()
+        # and it is the attention: against the plain formulas on the pages' own keys and values
+        plain = plain_decode_attention(q, cache, table, length, nq, nkv, d)
+        assert (got.double().cpu() - plain).abs().max() <= 2e-2 * plain.abs().max(), f"{seqs} sequences of {length}: not the plain attention"
     # one part: no scratch memory at all
     q, cache, table, positions = make_case(5, 4, 100, nq, nkv, d)
     want = ops.attention_mfma(q, cache, table, None, positions, nq, nkv, d, None, scale, 1, 0, 1, 1, False)

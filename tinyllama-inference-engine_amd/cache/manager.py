@@ -1,5 +1,5 @@
-"""The cache manager: pages of keys and values with a block table per request, in groups, and
-slots of fixed-size state.
+"""The cache manager: pages of what mixers keep per position (keys and values, for attention), with
+a block table per request, in groups, and slots of fixed-size state.
 
 reference: one request holds one slot, a whole [layers][max positions][kv width] region
 (src/cuda/model.cu:262-275, 615-617); `next_positions[slot]` says where its next token goes
@@ -7,13 +7,14 @@ reference: one request holds one slot, a whole [layers][max positions][kv width]
 Here a request holds pages instead, as many as its length needs, and a request slot that indexes
 the fixed-size state areas.
 
-Groups.  Runs of layers whose caches have the same need (every key kept, or a window of w
+Groups.  Runs of layers whose caches live equally long (every position kept, or a window of w
 positions) form a group.  A group has its own allocator and, per request, its own list of pages:
 entry b of the list is the page that holds positions b * page_size ... (b + 1) * page_size - 1.
 The page number is shared by all runs of the group: each run has its own pool tensor
-[pages, 2, kv heads, page_size * head_dim] (per page and kv head the keys lie as [row][dim], the values
-transposed, as [dim][row]), indexed by the same page number.  A windowed group
-gives a page back as soon as every position on it is out of every later token's window.
+[pages, *page shape], indexed by the same page number.  What a page looks like (how many planes,
+how many values per position, of which type) is the mixer's `CacheNeed`; how positions and values
+lie inside it is the mixer's own business, and nothing here knows of keys or values.  A windowed
+group gives a page back as soon as every position on it is out of every later token's window.
 
 Nothing is cleared when pages or slots come back: a kernel reads only rows that were written for
 the request that now owns the page, so what an earlier owner left cannot reach a result.
@@ -26,7 +27,7 @@ from typing import Hashable
 import torch
 
 from ..errors import EngineError, ErrorCode, invalid_argument, out_of_bounds, out_of_memory
-from ..parts.base import Binding, KVCacheNeed, StateNeed
+from ..parts.base import Binding, CacheNeed, StateNeed
 from .pages import PageAllocator
 
 ABSENT = -1     # in a request's page list: no page (not yet allocated, or given back by a window)
@@ -36,7 +37,7 @@ ABSENT = -1     # in a request's page list: no page (not yet allocated, or given
 class RunNeed:
     """What one run of a layer needs of the cache manager."""
     cache_of: int                       # the run whose cache this run reads (itself: it owns one)
-    kv: KVCacheNeed | None = None
+    cache: CacheNeed | None = None
     state: StateNeed | None = None
 
 
@@ -58,10 +59,12 @@ class RequestPages:
 class CacheManager:
     @staticmethod
     def page_bytes(needs: list[RunNeed], page_size: int, dtype: torch.dtype) -> int:
-        """Bytes that one more page costs over all runs that own a pool (keys and values)."""
-        itemsize = torch.empty((), dtype=dtype).element_size()
-        return sum(2 * need.kv.num_kv_heads * page_size * need.kv.head_dim * itemsize
-                   for run, need in enumerate(needs) if need.kv is not None and need.cache_of == run)
+        """Bytes that one more page costs over all runs that own a pool.  `dtype`: the type of
+        pools whose need names none."""
+        def itemsize(need):
+            return torch.empty((), dtype=need.dtype or dtype).element_size()
+        return sum(page_size * need.cache.values_per_position() * itemsize(need.cache)
+                   for run, need in enumerate(needs) if need.cache is not None and need.cache_of == run)
 
     def __init__(self, needs: list[RunNeed], page_size: int, num_pages: int, max_requests: int,
                  dtype: torch.dtype, device, max_positions: int | None = None, max_bytes: int | None = None):
@@ -94,25 +97,26 @@ class CacheManager:
         pools: dict[int, torch.Tensor] = {}
         group_of_run: dict[int, int] = {}
         for run, need in enumerate(needs):
-            if need.kv is not None and need.cache_of == run:
-                if need.kv.window not in group_of_window:
-                    group_of_window[need.kv.window] = len(self.groups)
-                    self.groups.append(PageGroup(need.kv.window, PageAllocator(num_pages)))
-                index = group_of_window[need.kv.window]
+            if need.cache is not None and need.cache_of == run:
+                if need.cache.window not in group_of_window:
+                    group_of_window[need.cache.window] = len(self.groups)
+                    self.groups.append(PageGroup(need.cache.window, PageAllocator(num_pages)))
+                index = group_of_window[need.cache.window]
                 self.groups[index].owners.append(run)
                 group_of_run[run] = index
-                # zeros once, at creation: rows that were never written then hold finite values
-                pools[run] = torch.zeros((num_pages, 2, need.kv.num_kv_heads, page_size * need.kv.head_dim),
-                                         dtype=dtype, device=device)
+                # zeros once, at creation: positions that were never written then hold finite values
+                pools[run] = torch.zeros((num_pages, *need.cache.page_shape(page_size)),
+                                         dtype=need.cache.dtype or dtype, device=device)
         for run, need in enumerate(needs):
             binding = Binding()
-            if need.kv is not None:
+            if need.cache is not None:
                 owner = need.cache_of
                 if owner not in pools:
                     raise invalid_argument(f"run {run} reads the cache of run {owner}, which owns none")
-                owner_need = needs[owner].kv
-                if (owner_need.num_kv_heads, owner_need.head_dim) != (need.kv.num_kv_heads, need.kv.head_dim):
-                    raise invalid_argument(f"run {run} reads the cache of run {owner}, whose heads have another shape")
+                owner_need = needs[owner].cache
+                if ((owner_need.planes, owner_need.width, owner_need.dtype)
+                        != (need.cache.planes, need.cache.width, need.cache.dtype)):
+                    raise invalid_argument(f"run {run} reads the cache of run {owner}, whose pages have another shape")
                 binding.group, binding.cache, binding.writes = group_of_run[owner], pools[owner], owner == run
             if need.state is not None:
                 area = torch.zeros((max_requests, *need.state.shape), dtype=need.state.dtype, device=device)

@@ -189,6 +189,8 @@ class LlamaConfig:
                                       "tied": self.tie_word_embeddings}),
             bos_token_id=self.bos_token_id,
             eos_token_id=self.eos_token_id,
+            # some writers of Llama checkpoints store the rotation's frequency table as a buffer
+            ignored_tensors=(r".*\.rotary_emb\.inv_freq",),
         )
         spec.validate()
         return spec

@@ -71,6 +71,10 @@ class ModelSpec:
     embedding_name: str = "model.embed_tokens.weight"
     final_norm_prefix: str = "model.norm."
     head_name: str = "lm_head.weight"
+    # tensors that this architecture's files may carry although no part reads them (buffers that
+    # some writers store): regular expressions matched against the whole name.  Anything else that
+    # the parts do not expect is an error.
+    ignored_tensors: tuple[str, ...] = ()
 
     def validate(self) -> None:
         from ..errors import invalid_config

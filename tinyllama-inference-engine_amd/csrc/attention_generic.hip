@@ -26,12 +26,20 @@ namespace tlie {
 // c % groups, and every group keeps a running maximum, sum and output of its own over its chunks,
 // in the order of their index; at the end the groups' results are put together in the order of
 // the groups.  Which keys meet in which sum, and in which order, depends on the positions alone.
+// seq_start (or null) with min_tokens: the step's cumulative token counts per sequence; tokens of
+// sequences that bring min_tokens tokens or more are then left to the tiled kernel below, which
+// is launched beside this one for the same step and leaves the others to this one.
 template <typename T, int CHUNK>
 __global__ void __launch_bounds__(256)
 attention_generic_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                          int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
-                         T* __restrict__ out, int nq, int nkv, int d, int page_size, int window, float scale) {
+                         T* __restrict__ out, int nq, int nkv, int d, int page_size, int window, float scale,
+                         const int* __restrict__ seq_start, int min_tokens) {
   constexpr int kGroups = 256 / CHUNK, kWavesPerGroup = CHUNK / 64;
+  if (seq_start != nullptr) {                      // (the same for the whole workgroup)
+    const int seq = token_seq[blockIdx.x];
+    if (seq_start[seq + 1] - seq_start[seq] >= min_tokens) return;
+  }
   extern __shared__ __attribute__((aligned(16))) float lds[];
   float* q_row = lds;                              // d
   float* prob = q_row + d;                         // 256: a group's probabilities of its current chunk
@@ -176,7 +184,7 @@ __global__ void __launch_bounds__(64 * kTiledWaves)
 attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ cache, const int* __restrict__ block_table,
                                int max_blocks, const int* __restrict__ token_seq, const int* __restrict__ positions,
                                T* __restrict__ out, int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
-                               int tokens_per_block, int heads_per_block) {
+                               int tokens_per_block, int heads_per_block, const int* __restrict__ seq_start, int min_tokens) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // rows of a multiple of 4 floats, so that four values are one LDS read, plus 4: a wave's lanes, each
   // on a row of its own, then spread over the banks
@@ -204,7 +212,11 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
 #pragma unroll
   for (int s = 0; s < kTiledSlots; ++s) {
     const int c = wave + kTiledWaves * s;
-    const bool live = c < ncols;
+    bool live = c < ncols;
+    if (live && seq_start != nullptr) {            // a token of a sequence that brings few tokens is the other kernel's
+      const int seq = token_seq[tok0 + c / nheads];
+      live = seq_start[seq + 1] - seq_start[seq] >= min_tokens;
+    }
     col_tok[s] = live ? c / nheads : -1;
     col_pos[s] = live ? positions[tok0 + col_tok[s]] : -1;
     col_lo[s] = live && window > 0 ? max(0, col_pos[s] - window + 1) : 0;
@@ -223,6 +235,10 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
     const int seq = token_seq[tok0 + run_first];
     int run_end = run_first + 1;
     while (run_end < ntok && token_seq[tok0 + run_end] == seq) ++run_end;
+    if (seq_start != nullptr && seq_start[seq + 1] - seq_start[seq] < min_tokens) {   // (the same for every thread)
+      run_first = run_end;
+      continue;
+    }
     // the keys the run's columns see: from the least lower bound to the last token's position
     int hi = -1, lo = 1 << 30;
     for (int t = run_first; t < run_end; ++t) {
@@ -301,7 +317,12 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
             run_max[g][s] = new_max;
             acc[g][s] *= alpha;
           }
-          // (a wave's lanes run in step: what one lane wrote to prob above, another may read below)
+          // what one lane wrote to prob above, another lane of the wave reads below: the writes are
+          // ordered before the reads for the compiler and the memory model (no instruction on this hardware,
+          // where a wave's LDS operations complete in order)
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+          __builtin_amdgcn_wave_barrier();
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
           if (lane < d) {
             const float* value = v_tile + lane * kValueStride;
 #pragma unroll
@@ -336,7 +357,7 @@ attention_generic_tiled_kernel(const T* __restrict__ q, const T* __restrict__ ca
 #pragma unroll
     for (int s = 0; s < kTiledSlots; ++s) {
       const int c = wave + kTiledWaves * s;
-      if (c >= ncols) continue;
+      if (c >= ncols || col_tok[s] < 0) continue;
       float top = -INFINITY;
 #pragma unroll
       for (int g = 0; g < 4; ++g) top = fmaxf(top, run_max[g][s]);
@@ -361,10 +382,18 @@ using namespace tlie;
 extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtype, const int* block_table,
                                       int max_blocks, const int* token_seq, const int* positions, void* out,
                                       int tokens, int nq, int nkv, int d, int page_size, int window, float scale,
-                                      int tiled, void* stream) {
+                                      int tiled, const int* seq_start, int min_tokens, void* stream) {
+  // tiled 0: the kernel of one (token, head) a workgroup; 1: the kernel that shares keys among a
+  // sequence's tokens (head sizes up to 64); 2: both, each token served by one of them: the second
+  // takes the sequences that bring min_tokens tokens or more (seq_start: int32 [sequences + 1], the
+  // step's cumulative token counts), the first the others.  A token gets the same bits from either.
   if (tokens <= 0 || nq <= 0 || nkv <= 0 || nq % nkv != 0 || d <= 0 || d > 256 || page_size <= 0 || max_blocks <= 0)
     return kBadArgument;
-  if (tiled && d <= 64 && (dtype == kF32 || dtype == kBF16)) {
+  if (tiled < 0 || tiled > 2 || (tiled == 2 && (seq_start == nullptr || min_tokens < 1))) return kBadArgument;
+  if (dtype != kF32 && dtype != kBF16) return kBadArgument;
+  if (d > 64) tiled = 0;
+  const int* select = tiled == 2 ? seq_start : nullptr;
+  if (tiled) {
     // (the same bits as the kernel below, for steps whose sequences bring several tokens each)
     const int G = nq / nkv;
     const int heads_per_block = G < kTiledCols ? G : kTiledCols;
@@ -375,12 +404,13 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
     if (dtype == kF32)
       hipLaunchKernelGGL((attention_generic_tiled_kernel<float>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const float*)q,
                          (const float*)cache, block_table, max_blocks, token_seq, positions, (float*)out, tokens, nq, nkv, d,
-                         page_size, window, scale, tokens_per_block, heads_per_block);
+                         page_size, window, scale, tokens_per_block, heads_per_block, select, min_tokens);
     else
       hipLaunchKernelGGL((attention_generic_tiled_kernel<bf16>), grid, dim3(64 * kTiledWaves), bytes, (hipStream_t)stream, (const bf16*)q,
                          (const bf16*)cache, block_table, max_blocks, token_seq, positions, (bf16*)out, tokens, nq, nkv, d,
-                         page_size, window, scale, tokens_per_block, heads_per_block);
-    return launch_status();
+                         page_size, window, scale, tokens_per_block, heads_per_block, select, min_tokens);
+    const int status = launch_status();
+    if (status != kOk || tiled == 1) return status;
   }
   const int chunk = d <= 64 ? 64 : (d <= 128 ? 128 : 256);
   const int groups = 256 / chunk;
@@ -389,7 +419,7 @@ extern "C" int tlie_attention_generic(const void* q, const void* cache, int dtyp
 #define TLIE_LAUNCH(T, CHUNK)                                                                                         \
   hipLaunchKernelGGL((attention_generic_kernel<T, CHUNK>), dim3(tokens, nq), dim3(256), lds, s, (const T*)q,           \
                      (const T*)cache, block_table, max_blocks, token_seq, positions, (T*)out, nq, nkv, d, page_size,   \
-                     window, scale)
+                     window, scale, select, min_tokens)
   if (dtype == kF32) {
     if (chunk == 64) TLIE_LAUNCH(float, 64); else if (chunk == 128) TLIE_LAUNCH(float, 128); else TLIE_LAUNCH(float, 256);
   } else if (dtype == kBF16) {

@@ -65,7 +65,7 @@ class Engine:
             if expect_sha256 is not None:
                 store.expect_sha256(expect_sha256)
             with device_memory_errors("the weights"):
-                weights = store.load(expected_tensors(self.spec), self.dtype, self.device)
+                weights = store.load(expected_tensors(self.spec), self.dtype, self.device, self.spec.ignored_tensors)
         else:
             if config is None or random_seed is None:
                 raise invalid_argument("without a model folder the engine needs a config and a random seed")
@@ -105,14 +105,16 @@ class Engine:
         self.cache.release(request)
 
     def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, trace: dict | None = None,
-             check_finite: bool = False) -> torch.Tensor:
+             check_finite: bool = False, trace_serving_route: bool = False) -> torch.Tensor:
         """One step of the model: see `ModelRunner.step`.  The logits are the caller's own (those
         of a step replayed from a recording are copied out of the recording's memory).  `trace`: a
-        dict that receives the step's intermediate tensors by the names of the reference's ModelTrace.
+        dict that receives the step's intermediate tensors by the names of the reference's ModelTrace,
+        all of them; with trace_serving_route a bfloat16 step of at most 16 tokens takes the route it
+        takes in serving (norms folded into the products) and leaves the names that exist there.
         check_finite: a NaN or an infinity among the logits is `numerical_error`, as the reference
         checks what it returns (src/cuda/model.cu:505-510); the step then waits for the device (the
         sampling kernel's test of a row runs over the logits and its marks are read)."""
-        logits = self.runner.step(entries, timings, trace=trace)
+        logits = self.runner.step(entries, timings, trace=trace, trace_serving_route=trace_serving_route)
         if check_finite and logits.shape[0] > 0:
             from ..ops import sample
             marks = sample(logits)
@@ -131,7 +133,8 @@ class Engine:
         steps' compute and transfer times, apart for steps that bring prompt tokens and steps that
         only decode (the keys of the reference's `generate`, app/cuda_reference.cu:216-224).
         `stats`: a dict that receives what the scheduler counted (steps, prompt and decoded tokens,
-        preemptions)."""
+        preemptions) and how many matrix products of this process fell from the vendor's library to the
+        plain kernel (`library_fallbacks`)."""
         scheduler = Scheduler(self.cache, max_tokens_per_step=max_tokens_per_step,
                               max_seqs_per_step=max_seqs_per_step or self.cache.max_requests, chunk_size=chunk_size,
                               max_positions=self.spec.max_positions, eos_token_id=self.spec.eos_token_id)
@@ -145,7 +148,9 @@ class Engine:
         try:
             self.run(scheduler, timings)
             if stats is not None:
+                from ..ops import library_fallbacks
                 stats.update(scheduler.stats)
+                stats["library_fallbacks"] = library_fallbacks()    # products that fell to the plain kernel so far (slow: should be 0)
         except BaseException:
             # a step raised (no request can move, a NaN in the logits, a device error): what this
             # call's requests hold goes back, so that the engine can be used again

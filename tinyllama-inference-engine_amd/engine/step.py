@@ -56,7 +56,13 @@ class GroupView:
 
 @dataclass
 class StepContext:
-    """Everything a part may need to know about the step, on the device (and on the host)."""
+    """Everything a part may need to know about the step, on the device (and on the host).
+
+    A step that is replayed from a recording is padded to the recording's size.  Padding tokens
+    (those from index seq_start[num_seqs] on) are token 0 at position 0, belong to no request
+    (`token_slot` -1), are written nowhere (slot maps -1) and their results are dropped; padding
+    sequences have `seq_slot` -1 and, in a step of portions, no tokens.  A part that keeps state
+    per request must change it only for tokens and sequences whose slot is not negative."""
     num_tokens: int
     num_seqs: int
     num_wanted: int
@@ -69,7 +75,8 @@ class StepContext:
     seq_start: torch.Tensor        # int32 [S + 1] first token of each sequence among the T
     seq_first_pos: torch.Tensor    # int32 [S] position of its first token
     seq_len: torch.Tensor          # int32 [S] length after this step
-    seq_slot: torch.Tensor         # int32 [S] request slot (row of the state areas)
+    seq_slot: torch.Tensor         # int32 [S] request slot (row of the state areas); -1: a padding sequence
+    token_slot: torch.Tensor       # int32 [T] request slot of the token's sequence; -1: a padding token
     want_rows: torch.Tensor        # int32 [num_wanted] token indices
     groups: list[GroupView]
     host: dict                     # the same arrays as numpy, by name
@@ -83,6 +90,9 @@ class StepContext:
     # replayed from a recording and takes no fused route), and the name's prefix for the layer that runs
     trace: dict | None = None
     trace_prefix: str = ""
+    # with a trace: False, every name of the trace is left (no norm is folded into a product); True, the step
+    # takes the route it would take without a trace and leaves the names that exist as tensors there
+    trace_serving_route: bool = False
     # what parts keep for the length of this step, under keys of their own (work lists that several
     # layers share, say); the step function never looks inside
     scratch: dict = field(default_factory=dict)
@@ -173,7 +183,7 @@ class ModelRunner:
 
     # ---- the step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry], timings: StepTimings | None = None, keep: bool = True,
-             trace: dict | None = None) -> torch.Tensor:
+             trace: dict | None = None, trace_serving_route: bool = False) -> torch.Tensor:
         """Runs exactly the tokens the entries bring, as one batch, from the cache that earlier
         steps left.  Returns float32 logits [wanted places, vocab] on the device, in the order of
         the entries and of each entry's `want`.  With `timings` the step is timed with events
@@ -181,7 +191,9 @@ class ModelRunner:
         a recording's memory, which the recording's next replay writes again (for a caller that
         has used them up by then); otherwise they are the caller's own.  trace: a dict that
         receives the step's intermediate tensors by name (see `DecoderModel.forward`); the step
-        is then launched kernel by kernel."""
+        is then launched kernel by kernel, and, unless trace_serving_route is set, on the route
+        that leaves every name (a bfloat16 step of few tokens would otherwise fold its norms into
+        its products)."""
         marks = None
         if timings is not None:
             import time
@@ -215,6 +227,7 @@ class ModelRunner:
                     raise invalid_argument("a token that is still on the device can only feed a replayed decode step")
                 ctx = self.build_context(entries)
                 ctx.trace = trace
+                ctx.trace_serving_route = trace_serving_route
                 if marks:
                     marks[1].record()
                 logits = self.model.forward(ctx, self.cache.bindings)
@@ -270,7 +283,7 @@ class DecodeGraph:
         self.widths = [max(1, (longest + cache.page_size - 1) // cache.page_size) for _ in cache.groups]
         layout = [("tokens", (bucket,)), ("positions", (bucket,)), ("token_seq", (bucket,)), ("no_slots", (bucket,)),
                   ("seq_start", (seqs + 1,)), ("seq_first_pos", (seqs,)), ("seq_len", (seqs,)), ("seq_slot", (seqs,)),
-                  ("want_rows", (seqs,)), ("token_source", (bucket,))]
+                  ("token_slot", (bucket,)), ("want_rows", (seqs,)), ("token_source", (bucket,))]
         for group, width in enumerate(self.widths):
             layout += [(f"block_table{group}", (seqs, width)), (f"slot_map{group}", (bucket,))]
         total = sum(int(np.prod(shape)) for _, shape in layout)
@@ -289,6 +302,8 @@ class DecodeGraph:
             self.host["want_rows"][:] = np.arange(bucket)
         self.host["no_slots"][:] = -1
         self.host["token_source"][:] = -1
+        self.host["seq_slot"][:] = -1
+        self.host["token_slot"][:] = -1
         self.token_source = views["token_source"]
         self.copied = torch.cuda.Event()                    # the last transfer of the pinned buffer has been made
         self.copy_pending = False
@@ -298,8 +313,8 @@ class DecodeGraph:
             num_tokens=bucket, num_seqs=seqs, num_wanted=seqs, max_new=1 if single else bucket, max_context=longest,
             tokens=views["tokens"], positions=views["positions"], token_seq=views["token_seq"], no_slots=views["no_slots"],
             seq_start=views["seq_start"], seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"],
-            seq_slot=views["seq_slot"], want_rows=views["want_rows"], groups=groups, host=self.host,
-            wants_all_rows=single,
+            seq_slot=views["seq_slot"], token_slot=views["token_slot"], want_rows=views["want_rows"], groups=groups,
+            host=self.host, wants_all_rows=single,
             compute_units=_compute_units(runner.device), tile_owner=None if single else self)
         self.graph = None
         self.logits = None
@@ -330,9 +345,11 @@ class DecodeGraph:
         held = [cache.held(entry.request) for entry in entries]
         positions = [info.length for info in held]
         stale = max(self._rows_filled, count)
-        for name in ("tokens", "positions", "seq_first_pos", "seq_slot"):
+        for name in ("tokens", "positions", "seq_first_pos"):
             host[name][count:stale] = 0
         host["seq_len"][count:stale] = 1
+        host["seq_slot"][count:stale] = -1                   # padding rows belong to no request: no state row is theirs
+        host["token_slot"][count:stale] = -1
         host["tokens"][:count] = [int(entry.tokens[0]) for entry in entries]
         host["token_source"][:count] = [-1 if entry.source is None else int(entry.source) for entry in entries]
         host["token_source"][count:stale] = -1
@@ -340,6 +357,7 @@ class DecodeGraph:
         host["seq_first_pos"][:count] = positions
         host["seq_len"][:count] = [position + 1 for position in positions]
         host["seq_slot"][:count] = [info.slot for info in held]
+        host["token_slot"][:count] = host["seq_slot"][:count]
         for group in range(len(cache.groups)):
             table, slots, known = host[f"block_table{group}"], host[f"slot_map{group}"], self._known[group]
             table[count:stale] = 0
@@ -467,7 +485,9 @@ class PortionGraph(DecodeGraph):
         host["seq_len"][:seqs] = [start + n for start, n in zip(first, counts)]
         host["seq_len"][seqs:] = 1
         host["seq_slot"][:seqs] = [cache.slot(entry.request) for entry in entries]
-        host["seq_slot"][seqs:] = 0
+        host["seq_slot"][seqs:] = -1                           # padding sequences belong to no request
+        host["token_slot"][:total] = np.repeat(host["seq_slot"][:seqs], counts)
+        host["token_slot"][total:] = -1
         want = [int(host["seq_start"][index]) + int(place) for index, entry in enumerate(entries) for place in entry.want]
         host["want_rows"][:len(want)] = want
         host["want_rows"][len(want):] = 0
@@ -511,6 +531,7 @@ def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> 
         "seq_slot": np.asarray([cache.slot(entry.request) for entry in entries], dtype=np.int32),
         "want_rows": want_rows,
     }
+    host["token_slot"] = np.repeat(host["seq_slot"], counts)
     group_shapes = []
     for group in range(len(cache.groups)):
         lists = [cache.page_list(entry.request, group) for entry in entries]
@@ -539,7 +560,7 @@ def build_context(cache: CacheManager, entries: Sequence[StepEntry], device) -> 
         max_context=int(host["seq_len"].max()), tokens=views["tokens"], positions=views["positions"],
         token_seq=views["token_seq"], no_slots=views["no_slots"], seq_start=views["seq_start"],
         seq_first_pos=views["seq_first_pos"], seq_len=views["seq_len"], seq_slot=views["seq_slot"],
-        want_rows=views["want_rows"], groups=groups, host=host,
+        token_slot=views["token_slot"], want_rows=views["want_rows"], groups=groups, host=host,
         wants_all_rows=bool(want_rows.size == total and np.array_equal(want_rows, np.arange(total))),
         compute_units=_compute_units(device))
 

@@ -57,7 +57,7 @@ class DecoderModel:
         needs = []
         for run in self.spec.runs:
             mixer = self.blocks[run.layer].mixer
-            needs.append(RunNeed(cache_of=run.cache_of, kv=mixer.cache_need(), state=mixer.state_need()))
+            needs.append(RunNeed(cache_of=run.cache_of, cache=mixer.cache_need(), state=mixer.state_need()))
         return needs
 
     def forward(self, ctx, bindings) -> torch.Tensor:
@@ -65,11 +65,13 @@ class DecoderModel:
         dict) the named tensors of the reference's ModelTrace are left there as float32 copies:
         "embedding", per run i "layer{i}.input_norm", ".attention_output", ".post_attention_norm",
         ".mlp_output", ".output", then "final_norm" and "logits" at the wanted rows
-        (src/model.cpp:98-231); a bfloat16 step of at most 16 tokens, which folds the norms into its
-        products, leaves the names that still exist as tensors on that route."""
+        (src/model.cpp:98-231).  A bfloat16 step of at most 16 tokens folds the norms into its
+        products when it serves; with a trace it does not, so that every name is left, unless
+        `ctx.trace_serving_route` asks for the serving route, which leaves the names that exist
+        as tensors there."""
         runs = self.spec.runs
         trace = getattr(ctx, "trace", None)
-        few = ops.few_rows_route(ctx.num_tokens, self.dtype)    # (also with a trace: it then shows the route that decoding takes)
+        few = ops.few_rows_route(ctx.num_tokens, self.dtype) and (trace is None or getattr(ctx, "trace_serving_route", False))
 
         def entry_norm(block):
             # a block may say which norm reads the residual first (its writer can then leave that

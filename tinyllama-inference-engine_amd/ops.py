@@ -17,6 +17,8 @@ from .errors import EngineError, ErrorCode, invalid_argument, invalid_shape
 
 F32, BF16 = 0, 1
 ROWS_MAX = 16          # the most rows the products take that fold in the layer's neighbouring arithmetic
+ATTENTION_MAX_HEAD_DIM = 256   # the largest head size that both attention kernels take
+GENERIC_TILED_MIN_TOKENS = 4   # a sequence's tokens in a step from which the plain attention shares its reads of the keys
 _CODES = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -222,12 +224,16 @@ def rope_cache(qkv: Product, positions: torch.Tensor, slot_map: torch.Tensor, in
 
 def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, token_seq: torch.Tensor,
                       positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
-                      window: int | None, scale: float, tiled: bool = False) -> torch.Tensor:
+                      window: int | None, scale: float, tiled: bool | int = False, seq_start: torch.Tensor | None = None,
+                      min_tokens: int = GENERIC_TILED_MIN_TOKENS) -> torch.Tensor:
     """Causal attention of every token over its sequence's cached keys; any number of tokens per
     sequence.  block_table: [sequences, max_blocks] pages; token_seq[t]: the token's row of it.
-    tiled: the step's sequences bring several tokens each (consecutive in the step, at consecutive
-    positions): neighbouring tokens then share each read of the keys (head sizes up to 64; the
-    result has the same bits either way)."""
+    tiled 1 (True): the step's sequences bring several tokens each (consecutive in the step, at
+    consecutive positions): neighbouring tokens then share each read of the keys (head sizes up to
+    64; the result has the same bits either way).  tiled 2: both kernels are launched and every token
+    is served by one of them: by the tiled one if its sequence brings `min_tokens` tokens or more
+    (seq_start: the step's cumulative token counts [sequences + 1], on the device), by the plain one
+    otherwise: for steps that mix portions of prompts with single tokens."""
     _device_tensor(q, "q", (torch.float32, torch.bfloat16))
     _device_tensor(cache, "cache", q.dtype)
     _device_tensor(block_table, "block_table", torch.int32)
@@ -241,13 +247,38 @@ def attention_generic(q: torch.Tensor, cache: torch.Tensor, block_table: torch.T
         raise invalid_shape("attention: block_table must be [sequences, max_blocks], token_seq and positions [tokens]")
     if num_heads % num_kv_heads != 0:
         raise invalid_shape("attention: the number of heads must be a multiple of the number of kv heads")
+    tiled = int(tiled)
+    if tiled == 2:
+        _device_tensor(seq_start, "seq_start", torch.int32)
+        if seq_start.dim() != 1 or seq_start.shape[0] != block_table.shape[0] + 1 or min_tokens < 1:
+            raise invalid_shape("attention: seq_start needs one entry more than the block table has rows, min_tokens at least 1")
+    elif tiled not in (0, 1):
+        raise invalid_argument("attention: tiled is 0, 1 or 2")
     out = torch.empty_like(q)
     _check(library().tlie_attention_generic(_ptr(q), _ptr(cache), dtype_code(q.dtype), _ptr(block_table),
                                             block_table.shape[1], _ptr(token_seq), _ptr(positions), _ptr(out), tokens,
                                             num_heads, num_kv_heads, head_dim, page_size,
-                                            int(window) if window else 0, ctypes.c_float(scale), 1 if tiled else 0, _stream()),
+                                            int(window) if window else 0, ctypes.c_float(scale), tiled,
+                                            _ptr(seq_start if tiled == 2 else None), int(min_tokens), _stream()),
            "attention_generic")
     return out
+
+
+def attention_generic_plan(ctx, head_dim: int) -> int:
+    """Which form of the plain attention kernel a step takes (the `tiled` of `attention_generic`): the
+    one that shares each read of the keys among a sequence's tokens pays from a few tokens a
+    sequence on, and costs dearly where a workgroup's 32 columns belong to many sequences of one
+    token (it walks each one's context in turn).  A launched step is decided from its host arrays;
+    a recorded step of portions, whose cut changes from replay to replay, launches both and lets
+    each sequence's token count on the device decide."""
+    if head_dim > 64 or ctx.max_new < GENERIC_TILED_MIN_TOKENS:
+        return 0
+    if ctx.tile_owner is not None:
+        return 2
+    starts = ctx.host["seq_start"]
+    counts = starts[1:] - starts[:-1]
+    many = int((counts >= GENERIC_TILED_MIN_TOKENS).sum())
+    return 1 if many == len(counts) else (2 if many else 0)
 
 
 def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, out_dtype: torch.dtype) -> Product:
@@ -270,7 +301,7 @@ def gemm_generic(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | Non
 
 
 # state: None (not tried), True, False (not there); fallbacks: products that took this library's plain kernel instead
-_library_gemm = {"state": None, "workspace": {}, "fallbacks": 0}
+_library_gemm = {"state": None, "workspace": {}, "fallbacks": 0, "warned": set()}
 LIBRARY_WORKSPACE_BYTES = 32 << 20
 
 
@@ -312,6 +343,14 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
     # where a library call that has not been tried may clear a workspace with a memset node)
     if x.shape[0] > 0:
         state["fallbacks"] += 1
+        shape = (x.shape[0], weight.shape[0], weight.shape[1])
+        if shape not in state["warned"]:
+            # said once per shape: nothing else shows why a prompt step is ten times slower than it should be
+            state["warned"].add(shape)
+            import warnings
+            why = "has no algorithm within its workspace for" if state["state"] else "is not available for"
+            warnings.warn(f"the vendor's matrix library {why} the bfloat16 product {shape[0]} x {shape[1]} x {shape[2]}; "
+                          f"it takes this library's plain 32-bit kernel, which is many times slower", stacklevel=2)
     return gemm_generic(x, weight, None, out_dtype).data
 
 
@@ -599,7 +638,7 @@ def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
 
 
 def attention_mfma_takes(dtype: torch.dtype, head_dim: int, page_size: int) -> bool:
-    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= 256 and page_size >= 16
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 0 < head_dim <= ATTENTION_MAX_HEAD_DIM and page_size >= 16
             and page_size & (page_size - 1) == 0)
 
 

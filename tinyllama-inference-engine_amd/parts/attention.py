@@ -17,7 +17,7 @@ from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..errors import invalid_config
 from ..registry import lookup, register
-from .base import Binding, KVCacheNeed, Mixer, PositionEncoding
+from .base import Binding, CacheNeed, Mixer, PositionEncoding
 from .linear import Linear
 
 
@@ -35,8 +35,12 @@ class Attention(Mixer):
         self.d = int(spec["head_dim"])
         self.bias = bool(spec.get("bias", False))
         self.window = spec.get("window")
-        if self.nq % self.nkv != 0:
-            raise invalid_config("attention: num_heads must be a multiple of num_kv_heads")
+        if self.nq <= 0 or self.nkv <= 0 or self.nq % self.nkv != 0:
+            raise invalid_config("attention: num_heads must be a positive multiple of num_kv_heads")
+        if not 0 < self.d <= ops.ATTENTION_MAX_HEAD_DIM:
+            # said here, where the model is built, not by the first step's launch
+            raise invalid_config(f"attention: head_dim {self.d} is beyond what the attention kernels take "
+                                 f"(1 to {ops.ATTENTION_MAX_HEAD_DIM})")
         if self.window is not None and int(self.window) <= 0:
             raise invalid_config("attention: a window must be a positive count of positions")
         position = spec.get("position") or PartSpec("none")
@@ -80,7 +84,10 @@ class Attention(Mixer):
         return self.qkv.takes_rows(rows)
 
     def cache_need(self):
-        return KVCacheNeed(self.nkv, self.d, int(self.window) if self.window is not None else None)
+        """A page holds two planes per kv head, [2, nkv, page_size * d]: the rotated keys as
+        [position][dim] and the values transposed, [dim][position], which is how the attention
+        kernels want them as matrix operands (`ops.rope_cache` writes them so)."""
+        return CacheNeed((2, self.nkv), self.d, int(self.window) if self.window is not None else None)
 
     def forward(self, x, ctx, binding: Binding, into=None):
         pages = ctx.groups[binding.group]
@@ -103,10 +110,9 @@ class Attention(Mixer):
             attended = ops.attention_mfma(q, binding.cache, pages.block_table, tiles, ctx.positions, self.nq, self.nkv,
                                           self.d, self.window, self.scale, nsplit, split_len, col_tiles, waves, shared)
         else:
-            # (sequences that bring four tokens or more on average: neighbouring tokens share the keys they read)
             attended = ops.attention_generic(q, binding.cache, pages.block_table, ctx.token_seq, ctx.positions, self.nq,
                                              self.nkv, self.d, self.window, self.scale,
-                                             tiled=ctx.num_tokens >= 4 * ctx.num_seqs)
+                                             tiled=ops.attention_generic_plan(ctx, self.d), seq_start=ctx.seq_start)
         return self.o(attended, into=into)
 
     def _apply_other_positions(self, qkv, ctx):

@@ -9,7 +9,7 @@ what the cache manager holds for it arrives in the `Binding`.
     Norm           forward(residual f32 [T, H]) -> [T, H] in the activation type
                    add_forward(residual, delta, rows=None): residual += delta, then forward
     Mixer          forward(x [T, H], ctx, binding) -> Product or tensor [T, H]
-                   cache_need() -> KVCacheNeed | None;  state_need() -> StateNeed | None
+                   cache_need() -> CacheNeed | None;  state_need() -> StateNeed | None
     FeedForward    forward(x [T, H], ctx) -> Product or tensor [T, H]
                    (both may opt into the fusions of steps of few rows, see Mixer below)
     PositionEncoding
@@ -29,12 +29,27 @@ from ..ops import NormedRows, Product, ResidualUpdated, as_product
 
 
 @dataclass(frozen=True)
-class KVCacheNeed:
-    """Pages of keys and values: [2, num_kv_heads, page_size * head_dim] per page.  `window`
-    None: every key stays; else only the last `window` positions are ever read again."""
-    num_kv_heads: int
-    head_dim: int
+class CacheNeed:
+    """Pages of whatever a mixer keeps per position.  A page of `page_size` positions is a tensor
+    of shape (*planes, page_size * width): in each of the prod(planes) planes, `width` values for
+    each of the page's positions.  How the positions and values lie inside a plane is the mixer's
+    own business (its kernels write and read the pages); the cache manager allocates and numbers
+    pages and looks at nothing inside them.  `dtype` None: the activation type of the run.
+    `window` None: every position stays; else only the last `window` positions are ever read again
+    (pages that no later token can see are given back)."""
+    planes: tuple[int, ...]
+    width: int
     window: int | None = None
+    dtype: torch.dtype | None = None
+
+    def page_shape(self, page_size: int) -> tuple[int, ...]:
+        return (*self.planes, page_size * self.width)
+
+    def values_per_position(self) -> int:
+        count = self.width
+        for plane in self.planes:
+            count *= plane
+        return count
 
 
 @dataclass(frozen=True)
@@ -48,7 +63,7 @@ class StateNeed:
 class Binding:
     """What the cache manager holds for one run of a layer."""
     group: int | None = None            # index of the page group (block table, slot map) in the step context
-    cache: torch.Tensor | None = None   # [pages, 2, nkv, page_size * d] of the run whose cache is read
+    cache: torch.Tensor | None = None   # [pages, *need.page_shape(page_size)] of the run whose cache is read
     writes: bool = True                 # this run owns the cache and writes the step's keys and values
     state: torch.Tensor | None = None   # [request slots, *shape] for a mixer with state of its own
 
@@ -115,7 +130,7 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    def cache_need(self) -> KVCacheNeed | None:
+    def cache_need(self) -> CacheNeed | None:
         return None
 
     def state_need(self) -> StateNeed | None:
@@ -146,5 +161,5 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
-__all__ = ["KVCacheNeed", "StateNeed", "Binding", "Part", "Norm", "PositionEncoding", "Mixer", "FeedForward",
+__all__ = ["CacheNeed", "StateNeed", "Binding", "Part", "Norm", "PositionEncoding", "Mixer", "FeedForward",
            "Product", "as_product", "NormedRows", "ResidualUpdated", "ResidualTarget"]

@@ -64,13 +64,14 @@ class PreNormBlock:
         their results into the residual themselves; otherwise the norm kernels do both.
         A step that keeps a trace (`ctx.trace`, a dict) leaves there, under `ctx.trace_prefix`, the
         five tensors the reference's ModelTrace keeps per layer
-        (src/model.cpp:136-138,176-177,184-185,200-201,204-205), as float32 copies; on the route of
-        few rows, which it takes as a step without a trace would, those that still exist there:
-        "attention_output" and "mlp_output" (what the part added into the residual: the residual
-        after it minus the residual before) and "output" (the normed inputs are folded away)."""
+        (src/model.cpp:136-138,176-177,184-185,200-201,204-205), as float32 copies, and takes the route
+        on which all five exist; with `ctx.trace_serving_route` a step of few rows takes the route
+        it takes without a trace and leaves those that still exist there: "attention_output" and
+        "mlp_output" (what the part added into the residual: the residual after it minus the
+        residual before) and "output" (the normed inputs are folded away)."""
         trace = getattr(ctx, "trace", None)
         rows = residual.shape[0]
-        few = ops.few_rows_route(rows, self.dtype)
+        few = ops.few_rows_route(rows, self.dtype) and (trace is None or getattr(ctx, "trace_serving_route", False))
         if trace is not None and not few:
             return self._forward_traced(residual, pending, ctx, binding)
 

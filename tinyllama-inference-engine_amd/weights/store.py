@@ -22,9 +22,6 @@ from ..config.spec import TensorSpec
 from ..errors import EngineError, ErrorCode
 from .safetensors_io import SafetensorsFile
 
-# buffers that some writers store although they are no weights
-_IGNORED = (re.compile(r".*\.rotary_emb\.inv_freq$"),)
-
 
 class WeightStore:
     """All safetensors files of a model folder behind one `get(name)`."""
@@ -97,12 +94,16 @@ class WeightStore:
             raise EngineError(ErrorCode.INVALID_SHAPE, f"required tensor is missing: {name}")
         return self._where[name].tensor(name)
 
-    def validate(self, specs: Iterable[TensorSpec]) -> None:
+    def validate(self, specs: Iterable[TensorSpec], ignored: Iterable[str] = ()) -> None:
+        """ignored: patterns (regular expressions, matched against the whole name) of tensors
+        that the architecture's files may carry although no part reads them (the model's
+        specification names them: `ModelSpec.ignored_tensors`)."""
         specs = list(specs)
+        patterns = [re.compile(pattern) for pattern in ignored]
         expected = {spec.name: spec for spec in specs}
         missing = [spec.name for spec in specs if not spec.optional and spec.name not in self._where]
         unexpected = [name for name in self.names()
-                      if name not in expected and not any(pattern.match(name) for pattern in _IGNORED)]
+                      if name not in expected and not any(pattern.fullmatch(name) for pattern in patterns)]
         wrong = []
         for spec in specs:
             if spec.name in self._where and tuple(self.shape(spec.name)) != tuple(spec.shape):
@@ -118,14 +119,15 @@ class WeightStore:
             raise EngineError(ErrorCode.INVALID_SHAPE,
                               f"weights in {self.model_dir} do not fit the model — " + " | ".join(parts))
 
-    def load(self, specs: Iterable[TensorSpec], dtype: torch.dtype, device) -> dict[str, torch.Tensor]:
+    def load(self, specs: Iterable[TensorSpec], dtype: torch.dtype, device,
+             ignored: Iterable[str] = ()) -> dict[str, torch.Tensor]:
         """Validates, then uploads every required tensor, in its kept precision.  A tensor the
         model marks optional (a tied head's matrix that some files still carry) is checked when
         present and not uploaded: no part reads it.  A matrix stored in 32-bit stays 32-bit also in
         a bfloat16 run (its products then go to the true 32-bit kernel, at a fraction of the
         speed): that is said once, as a warning, because nothing else shows it."""
         specs = list(specs)
-        self.validate(specs)
+        self.validate(specs, ignored)
         out, wide = {}, []
         for spec in specs:
             if spec.name in self._where and not spec.optional:
