@@ -456,6 +456,46 @@ def test_library_mm_takes_the_library_for_many_rows(shape):
     assert rel_err(got32[:2].cpu(), want[:2].cpu()) < 5e-5
 
 
+@pytest.mark.parametrize("shape", [(1, 4, 64), (65, 260, 128), (130, 2560, 2048), (300, 96, 5632), (257, 1000, 192), (2048, 132, 64)])
+def test_gemm_tiles_against_the_plain_product(shape):
+    """This library's own product of many rows (tiles of 128 x 128 on the matrix cores), at sizes that
+    are no multiple of its tiles: bfloat16 and float32 results against the float64 product."""
+    from tlie_amd import ops
+    m, n, k = shape
+    torch.manual_seed(m * 7 + n)
+    x = torch.randn(m, k, device=DEV).bfloat16()
+    w = (torch.randn(n, k, device=DEV) / math.sqrt(k)).bfloat16()
+    want = plain_linear(x.cpu().double(), w.cpu().double())
+    assert rel_err(ops.gemm_tiles(x, w, torch.float32).cpu(), want) < 5e-6
+    got = ops.gemm_tiles(x, w)
+    assert got.dtype == torch.bfloat16 and rel_err(got.cpu(), want) < 6e-3                 # one rounding to bfloat16
+    for bad_n, bad_k in ((n + 1, k), (n, k + 8)):
+        with pytest.raises(ops.EngineError):
+            ops.gemm_tiles(torch.zeros(m, bad_k, device=DEV).bfloat16(), torch.zeros(bad_n, bad_k, device=DEV).bfloat16())
+
+
+def test_library_mm_without_the_library_takes_the_tiled_kernel_and_says_so(monkeypatch):
+    """Where the vendor's library cannot be called, a product of many rows takes this library's tiled
+    kernel (or, for sizes that one refuses, the plain 32-bit kernel), counts it and warns once per shape."""
+    import warnings
+    from tlie_amd import ops
+    torch.manual_seed(3)
+    x = torch.randn(200, 256, device=DEV).bfloat16()
+    w = (torch.randn(96, 256, device=DEV) / 16).bfloat16()
+    odd = (torch.randn(97, 256, device=DEV) / 16).bfloat16()                  # 97 rows: not the tiled kernel's
+    ops.library_mm(x, w)                                                     # (the library is set up, if it is there)
+    monkeypatch.setitem(ops._library_gemm, "state", False)
+    monkeypatch.setitem(ops._library_gemm, "warned", set())
+    before = ops.library_fallbacks()
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        got, again, plain = ops.library_mm(x, w), ops.library_mm(x, w, torch.float32), ops.library_mm(x, odd)
+    assert ops.library_fallbacks() == before + 3
+    assert len(caught) == 2 and "tiled kernel" in str(caught[0].message) and "32-bit kernel" in str(caught[1].message)
+    assert torch.equal(got, ops.gemm_tiles(x, w)) and torch.equal(again, ops.gemm_tiles(x, w, torch.float32))
+    assert rel_err(plain.cpu(), plain_linear(x.cpu().double(), odd.cpu().double())) < 6e-3
+
+
 def test_gemm_skinny_refuses():
     from tlie_amd import EngineError, ops
     w = torch.randn(32, 64, device=DEV).bfloat16()

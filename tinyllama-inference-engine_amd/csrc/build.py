@@ -16,7 +16,7 @@ import time
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["elementwise.hip", "rope_cache.hip", "attention_generic.hip", "attention_mfma.hip", "gemm_generic.hip",
-           "gemm_skinny.hip", "gemm_rows.hip", "sampling.hip", "library_gemm.hip", "probes.hip"]
+           "gemm_skinny.hip", "gemm_rows.hip", "gemm_tiles.hip", "sampling.hip", "library_gemm.hip", "probes.hip"]
 HEADERS = ["common.h", "no_alloc.h"]
 LIBRARY = "libtlie_hip.so"
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared",

@@ -338,9 +338,11 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
         if status != -3:
             _check(status, "library_gemm")
     # where the library cannot be called directly (its file is not beside torch, or it has no
-    # algorithm for the shape) this library's plain kernel makes the product: one route, recorded or
-    # not, so that a step gives the same bits replayed and launched (slow, and safe inside a recording,
-    # where a library call that has not been tried may clear a workspace with a memset node)
+    # algorithm for the shape) this library's own kernels make the product: the tiled one on the matrix
+    # cores (some two thirds of the vendor's speed) for sizes it takes, else the plain 32-bit one (many
+    # times slower); one route, recorded or not, so that a step gives the same bits replayed and launched
+    # (and safe inside a recording, where a library call that has not been tried may clear a workspace
+    # with a memset node)
     if x.shape[0] > 0:
         state["fallbacks"] += 1
         shape = (x.shape[0], weight.shape[0], weight.shape[1])
@@ -349,14 +351,42 @@ def library_mm(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = t
             state["warned"].add(shape)
             import warnings
             why = "has no algorithm within its workspace for" if state["state"] else "is not available for"
+            how = ("this library's tiled kernel, at some two thirds of the speed" if gemm_tiles_takes(weight)
+                   else "this library's plain 32-bit kernel, which is many times slower")
             warnings.warn(f"the vendor's matrix library {why} the bfloat16 product {shape[0]} x {shape[1]} x {shape[2]}; "
-                          f"it takes this library's plain 32-bit kernel, which is many times slower", stacklevel=2)
+                          f"it takes {how}", stacklevel=2)
+    if gemm_tiles_takes(weight):
+        return gemm_tiles(x, weight, out_dtype)
     return gemm_generic(x, weight, None, out_dtype).data
 
 
+def gemm_tiles_takes(weight: torch.Tensor) -> bool:
+    return weight.dtype == torch.bfloat16 and weight.shape[1] % 64 == 0 and weight.shape[0] % 4 == 0
+
+
+def gemm_tiles(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """y = x . W^T of bfloat16 operands on this library's own tiled kernel for many rows (tiles of 128
+    rows of W by 128 tokens on the matrix cores): what `library_mm` runs where the vendor's library
+    cannot be called.  The inner size a multiple of 64, W's rows a multiple of 4; y bfloat16 or float32."""
+    _device_tensor(x, "x", torch.bfloat16)
+    _device_tensor(weight, "weight", torch.bfloat16)
+    if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+        raise invalid_shape(f"gemm_tiles: x {list(x.shape)} and weight {list(weight.shape)} do not fit")
+    if out_dtype not in (torch.bfloat16, torch.float32):
+        raise EngineError(ErrorCode.INVALID_DTYPE, f"gemm_tiles gives bfloat16 or float32, not {out_dtype}")
+    if not gemm_tiles_takes(weight):
+        raise invalid_argument("gemm_tiles takes an inner size that is a multiple of 64 and a multiple of 4 of rows of W")
+    out = torch.empty((x.shape[0], weight.shape[0]), dtype=out_dtype, device=x.device)
+    if x.shape[0] == 0:
+        return out
+    _check(library().tlie_gemm_tiles(_ptr(x), _ptr(weight), _ptr(out), int(out_dtype == torch.float32), x.shape[0],
+                                     weight.shape[0], x.shape[1], _stream()), "gemm_tiles")
+    return out
+
+
 def library_fallbacks() -> int:
-    """How many products `library_mm` has made with the plain kernel because the vendor's library
-    was not there or offered nothing for the shape (each many times slower)."""
+    """How many products `library_mm` has made with this library's own kernels because the vendor's
+    library was not there or offered nothing for the shape (each slower, some many times)."""
     return _library_gemm["fallbacks"]
 
 
