@@ -117,7 +117,7 @@ def time_prefill(engine, torch, tokens, vocab, repeats=3):
     return best
 
 
-def run_workload(engine, torch, workload, vocab, budget, chunk, slice_steps=8):
+def run_workload(engine, torch, workload, vocab, budget, chunk, slice_steps=8, prompt_cap=None):
     """A whole workload through the scheduler and the engine's loop, timed in slices of a few
     steps.  Returns the record's `value` parts and what the scheduler and the cache counted.
     serving: 64 requests at once, prompts of 128 to 2048 random tokens (or as many as leave the
@@ -133,7 +133,8 @@ def run_workload(engine, torch, workload, vocab, budget, chunk, slice_steps=8):
     else:
         shapes = [(rng.randint(32, 128), 256) for _ in range(56)] + [(8192 - 16, 16) for _ in range(8)]   # 8192 positions each
     scheduler = Scheduler(engine.cache, max_tokens_per_step=budget, max_seqs_per_step=len(shapes), chunk_size=chunk,
-                          max_positions=engine.spec.max_positions, eos_token_id=engine.spec.eos_token_id)
+                          max_positions=engine.spec.max_positions, eos_token_id=engine.spec.eos_token_id,
+                          prompt_tokens_beside_decodes=prompt_cap)
     requests = [Request(id=(workload, index), prompt=torch.randint(0, vocab, (length,), generator=generator).tolist(),
                         params=SamplingParams(max_tokens=new)) for index, (length, new) in enumerate(shapes)]
     for request in requests:
@@ -179,6 +180,8 @@ def main() -> int:
                              "continuously; mixed: 8 prompts of 8192 tokens in portions beside 56 short decode streams "
                              "(needs a shape with 8192 positions); each prints a record of its own")
     parser.add_argument("--token-budget", type=int, default=2048, help="tokens a step of a workload may hold")
+    parser.add_argument("--prompt-cap", type=int, default=0,
+                        help="workloads: the most prompt tokens in a step that also holds decoding requests (0: what the budget leaves)")
     parser.add_argument("--kernels", nargs="?", const="", default=None, metavar="NAME",
                         help="time the kernels of a decode step (--batch, --context) and of a prompt step one by one at the "
                              "shape's layer sizes, each inside a replayed recording that walks through copies of its weights; "
@@ -215,11 +218,13 @@ def main() -> int:
         live = 64 * (2048 + 256) if args.workload == "serving" else 8 * (8192 + 64) + 56 * (128 + 256 + 64)
         engine = Engine(None, dtype=args.dtype, config=cfg, random_seed=0, max_tokens=live, page_size=16, max_requests=65)
         chunk = None if args.workload == "serving" else 512
-        run_workload(engine, torch, args.workload, vocab, args.token_budget, chunk)            # warms up (recordings, plans)
-        got = run_workload(engine, torch, args.workload, vocab, args.token_budget, chunk)
+        cap = args.prompt_cap or None
+        run_workload(engine, torch, args.workload, vocab, args.token_budget, chunk, prompt_cap=cap)   # warms up (recordings, plans)
+        got = run_workload(engine, torch, args.workload, vocab, args.token_budget, chunk, prompt_cap=cap)
         print(json.dumps({"metric": f"total tok/s, {args.workload} workload ({model_name})", "value": got["tokens"] / got["seconds"],
                           "unit": "tokens/s", "generated_per_s": got["generated"] / got["seconds"], "seconds": got["seconds"],
                           "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "token_budget": args.token_budget,
+                          "prompt_tokens_beside_decodes": args.prompt_cap or None,
                           "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
                           **{key: got[key] for key in ("steps", "preemptions", "peak_pages_frac", "ms_step_with_prompts",
                                                        "ms_step_decode_only")}}))
@@ -283,12 +288,13 @@ def main() -> int:
             points[f"decode_b{batch}_frac"] = step_bytes(cfg, itemsize, batch, args.context, steps) / (seconds / steps) / HBM_PEAK
         # a short prompt: its step is replayed from a recording (the long one's is launched kernel by kernel)
         points["prefill_256"] = 256 / time_prefill(engine, torch, 256, vocab)
-        # the workload of a prompt of 128 tokens and 128 generated ones, at the record's batch
+        # the workload of a prompt of 128 tokens and 128 generated ones, at the record's batch and at 1 and 64
         warm = 8
         timed = 128 - warm - 1
-        seconds = median_decode(engine, args.batch, 256, timed, warm, vocab, args.repeats)
-        points[f"decode_b{args.batch}_prompt128"] = args.batch * timed / seconds
-        points[f"decode_b{args.batch}_prompt128_frac"] = step_bytes(cfg, itemsize, args.batch, 256, timed) / (seconds / timed) / HBM_PEAK
+        for batch in sorted({args.batch, 1, 64}):
+            seconds = median_decode(engine, batch, 256, timed, warm, vocab, args.repeats)
+            points[f"decode_b{batch}_prompt128"] = batch * timed / seconds
+            points[f"decode_b{batch}_prompt128_frac"] = step_bytes(cfg, itemsize, batch, 256, timed) / (seconds / timed) / HBM_PEAK
         del engine
         torch.cuda.empty_cache()
         if args.dtype == "bfloat16" and args.shape == "tinyllama":
@@ -337,6 +343,19 @@ def main() -> int:
                 points[key + "_ms_step_with_prompts"] = got["ms_step_with_prompts"]
                 points[key + "_ms_step_decode_only"] = got["ms_step_decode_only"]
                 points[key + "_preemptions"] = got["preemptions"]
+                if workload == "mixed":
+                    # the other end of the trade: prompts get at most 256 tokens in a step that also decodes, so
+                    # the 56 decoding streams wait less for each of their tokens and the long prompts take longer
+                    run_workload(other, torch, workload, larger["vocab_size"], 2048, chunk, prompt_cap=256)
+                    got = run_workload(other, torch, workload, larger["vocab_size"], 2048, chunk, prompt_cap=256)
+                    points[key + "_cap256_tok_s"] = got["tokens"] / got["seconds"]
+                    points[key + "_cap256_generated_tok_s"] = got["generated"] / got["seconds"]
+                    points[key + "_cap256_ms_step_with_prompts"] = got["ms_step_with_prompts"]
+                    # and decoding at the model's longest context, 8192 positions, at the record's batch
+                    steps = 24
+                    seconds = median_decode(other, args.batch, 8192, steps, 4, larger["vocab_size"], args.repeats)
+                    points[f"{shape}_decode_b{args.batch}_ctx8192"] = args.batch * steps / seconds
+                    points[f"{shape}_decode_b{args.batch}_ctx8192_frac"] = step_bytes(larger, 2, args.batch, 8192, steps) / (seconds / steps) / HBM_PEAK
                 del other
                 torch.cuda.empty_cache()
         record["points"] = points

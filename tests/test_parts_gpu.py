@@ -401,9 +401,20 @@ def register_recorded_state_toy():
     request slots from the device (`token_slot`, `seq_slot`) and moves the state of live rows
     only: a recorded step's padding has slot -1."""
     from tlie_amd.config import LayerSpec, ModelSpec, PartSpec, Run, TensorSpec
-    from tlie_amd.parts import Mixer, StateNeed
+    from tlie_amd.parts import Mixer, PositionEncoding, StateNeed
     from tlie_amd.parts.linear import Linear
     from tlie_amd.registry import register
+
+    @register("position_encoding", "toy_recorded_scale_by_position")
+    class RecordedScaleByPosition(PositionEncoding):
+        """Not a rotation: keys are scaled by 1 / (1 + position / 64), with tensor operations whose
+        sizes depend on the token count alone, so it says that it may be recorded (and the attention
+        around it then may be too)."""
+        graph_safe = True
+
+        def apply_qk(self, q, k, positions):
+            scale = (1.0 / (1.0 + positions.float() / 64.0))[:, None, None]
+            return q, (k.float() * scale).to(k.dtype)
 
     @register("mixer", "toy_recorded_running_mean")
     class RecordedRunningMean(Mixer):
@@ -424,7 +435,9 @@ def register_recorded_state_toy():
             count = x.shape[0]
             live = ctx.token_slot >= 0
             rows = ctx.token_slot.long().clamp(min=0)
-            values = x.float() * live[:, None]                       # padding tokens count for nothing
+            # padding tokens count for nothing (their rows of x may hold anything, not even finite values:
+            # no attention tile serves them, so they are taken out, not multiplied by zero)
+            values = torch.where(live[:, None], x.float(), torch.zeros((), device=x.device))
             index = torch.arange(count, device=x.device)
             before = (ctx.token_seq[:, None] == ctx.token_seq[None, :]) & (index[None, :] <= index[:, None]) & live[None, :]
             sums = (before[:, :, None] * values[None, :, :]).sum(dim=1) + binding.state[rows]
@@ -455,7 +468,7 @@ def register_recorded_state_toy():
             norm = PartSpec("rms_norm", {"size": self.hidden_size, "eps": self.eps})
             attention = PartSpec("attention", {"hidden_size": self.hidden_size, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
                                                "bias": False, "window": None,
-                                               "position": PartSpec("rotary", {"head_dim": 16, "theta": 100.0})})
+                                               "position": PartSpec("toy_recorded_scale_by_position")})
             mean = PartSpec("toy_recorded_running_mean", {"hidden_size": self.hidden_size})
             mlp = PartSpec("gated_mlp", {"hidden_size": self.hidden_size, "intermediate_size": 40, "activation": "silu"})
             layers = (LayerSpec("model.layers.0.", "pre_norm", attention, mlp, norm, norm),
@@ -476,7 +489,11 @@ def plain_recorded_state_forward(raw, w, tokens):
         return plain_linear(plain_silu_mul(plain_linear(normed, w[p + "mlp.gate_proj.weight"]),
                                            plain_linear(normed, w[p + "mlp.up_proj.weight"])), w[p + "mlp.down_proj.weight"])
     p = "model.layers.0."
-    x = x + plain_attention_part(plain_rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", 2, 1, 16, 100.0, None, False)
+    normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)
+    q = plain_linear(normed, w[p + "self_attn.q_proj.weight"]).view(count, 2, 16)
+    k = plain_linear(normed, w[p + "self_attn.k_proj.weight"]).view(count, 1, 16) / (1.0 + torch.arange(count).double() / 64.0)[:, None, None]
+    v = plain_linear(normed, w[p + "self_attn.v_proj.weight"]).view(count, 1, 16)
+    x = x + plain_linear(plain_attention(q, k, v).reshape(count, 32), w[p + "self_attn.o_proj.weight"])
     x = x + mlp(x, p)
     p = "model.layers.1."
     normed = plain_rms_norm(x, w[p + "input_layernorm.weight"], eps)

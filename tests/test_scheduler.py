@@ -20,8 +20,9 @@ def fake_token(tokens):
     return (sum(tokens) * 31 + len(tokens) * 7) % 97
 
 
-def drive(cache, scheduler, log=None, max_steps=500):
-    """Runs plans against the cache manager as the engine loop does."""
+def drive(cache, scheduler, log=None, max_steps=500, finish=True):
+    """Runs plans against the cache manager as the engine loop does, to the end (or, with
+    finish=False, for max_steps steps)."""
     for _ in range(max_steps):
         if not scheduler.has_work():
             return
@@ -41,7 +42,8 @@ def drive(cache, scheduler, log=None, max_steps=500):
         sampled = [fake_token(item.request.tokens[:item.first + item.count]) for item in plan if item.samples]
         scheduler.update(plan, sampled)
         cache.check()
-    raise AssertionError("did not finish")
+    if finish:
+        raise AssertionError("did not finish")
 
 
 def expected_output(prompt, count):
@@ -79,6 +81,32 @@ def test_decodes_first_then_fills_with_prompt_portions_fifo():
     assert log[2] == [("a", 4, 1, True), ("b", 8, 3, True), ("c", 0, 2, True)]
     for request in (a, b, c):
         assert request.generated == expected_output(request.prompt, request.params.max_tokens)
+
+
+def test_prompts_beside_decoding_requests_can_be_capped():
+    """A step's time grows with its prompt tokens and its decoding requests wait for all of it: with
+    a cap, prompts get at most so many tokens in a step that also decodes, and the whole budget in a
+    step that does not.  The outputs do not change."""
+    def run(cap):
+        cache, scheduler = make(max_tokens_per_step=16, num_pages=32, prompt_tokens_beside_decodes=cap)
+        a = Request("a", [1, 2, 3], SamplingParams(max_tokens=6))
+        b = Request("b", list(range(10, 40)), SamplingParams(max_tokens=2))
+        scheduler.add(a)
+        log = []
+        drive(cache, scheduler, log, max_steps=1, finish=False)     # "a" is decoding when "b" arrives
+        scheduler.add(b)
+        drive(cache, scheduler, log)
+        assert a.generated == expected_output(a.prompt, 6) and b.generated == expected_output(b.prompt, 2)
+        return log
+    free = run(None)
+    assert free[1] == [("a", 3, 1, True), ("b", 0, 15, False)] and free[2] == [("a", 4, 1, True), ("b", 15, 15, True)]
+    capped = run(4)
+    assert capped[1] == [("a", 3, 1, True), ("b", 0, 4, False)] and capped[2] == [("a", 4, 1, True), ("b", 4, 4, False)]
+    # once "a" has finished (its fifth decode step is the trace's sixth), the prompt takes the whole budget again
+    alone = [step for step in capped if [item[0] for item in step] == ["b"]]
+    assert alone and alone[0][0][2] == 10                      # the 10 tokens that were left, in one step
+    with pytest.raises(EngineError):
+        make(prompt_tokens_beside_decodes=0)
 
 
 def test_admission_waits_for_a_slot():
@@ -246,7 +274,8 @@ def drive_a_step_behind(cache, scheduler, max_steps=500):
         else:
             scheduler.update(plan, sampled)
         cache.check()
-    raise AssertionError("did not finish")
+    if finish:
+        raise AssertionError("did not finish")
 
 
 def test_tokens_may_arrive_a_step_late():

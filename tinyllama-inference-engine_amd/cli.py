@@ -19,7 +19,8 @@ Options (after the positionals): --dtype bfloat16|float32, --temperature T, --to
 (the reference's request options of the same names, app/server.cpp:601-613); the cache and the
 scheduler: --max-cache-tokens N (positions the page pool holds), --page-size P, --max-requests R
 (request slots), --max-tokens-per-step T (a step's token budget), --chunk-size C (the most tokens of
-one prompt in a step); `batch`: --batch N (default 4), --min-ratio X (fail below this speed-up).
+one prompt in a step), --prompt-tokens-beside-decodes N (the most prompt tokens in a step that also
+decodes); `batch`: --batch N (default 4), --min-ratio X (fail below this speed-up).
 """
 from __future__ import annotations
 
@@ -37,7 +38,7 @@ USAGE = ("usage: tinyllama_amd generate MODEL_DIR PROMPT MAX_TOKENS [GOLDEN_JSON
          "       tinyllama_amd random MODEL_DIR CONFIG_JSON SEED\n"
          "options: [--dtype bfloat16|float32] [--temperature T] [--top-p P] [--seed S] [--expect-sha256 HEX]\n"
          "         [--max-cache-tokens N] [--page-size P] [--max-requests R] [--max-tokens-per-step T] [--chunk-size C]\n"
-         "         [--prompts-file FILE] [--batch N] [--min-ratio X]\n")
+         "         [--prompt-tokens-beside-decodes N] [--prompts-file FILE] [--batch N] [--min-ratio X]\n")
 
 
 def parse_integer(text: str, name: str, minimum: int) -> int:
@@ -71,7 +72,7 @@ def _engine(args, positions: int, requests: int = 1):
     """positions: what the live requests hold at most when the caller names no pool size (each
     request's share rounded up to whole pages)."""
     from .engine import Engine
-    for name in ("page_size", "max_requests", "max_cache_tokens", "max_tokens_per_step", "chunk_size"):
+    for name in ("page_size", "max_requests", "max_cache_tokens", "max_tokens_per_step", "chunk_size", "prompt_tokens_beside_decodes"):
         if getattr(args, name) < 0:
             raise invalid_argument(f"--{name.replace('_', '-')} must be positive")
     page_size = args.page_size or 16
@@ -114,7 +115,8 @@ def command_generate(args) -> int:
     timings, stats = {}, {}
     outputs = engine.generate(prompts, max_tokens=max_tokens, temperature=args.temperature, top_p=args.top_p,
                               seed=args.seed, timings=timings, stats=stats,
-                              max_tokens_per_step=args.max_tokens_per_step or 2048, chunk_size=args.chunk_size or None)
+                              max_tokens_per_step=args.max_tokens_per_step or 2048, chunk_size=args.chunk_size or None,
+                              prompt_tokens_beside_decodes=args.prompt_tokens_beside_decodes or None)
     generated = outputs[0]
     elapsed = (time.perf_counter() - started) * 1e3
     if len(args.rest) > 1:
@@ -320,6 +322,7 @@ def main(argv=None) -> int:
     parser.add_argument("--max-requests", type=int, default=0)
     parser.add_argument("--max-tokens-per-step", type=int, default=0)
     parser.add_argument("--chunk-size", type=int, default=0)
+    parser.add_argument("--prompt-tokens-beside-decodes", type=int, default=0)
     parser.add_argument("--prompts-file", default=None)
     parser.add_argument("--batch", type=int, default=4)
     parser.add_argument("--min-ratio", type=float, default=0.0)

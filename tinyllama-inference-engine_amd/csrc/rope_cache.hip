@@ -87,13 +87,19 @@ __global__ void rope_cache_wide_kernel(const D* __restrict__ qkv, const int* __r
   float* cosines = lds;                  // half
   float* sines = cosines + half;         // half
   const int t = blockIdx.x;
+  const int heads = nq + 2 * nkv, per_head = d / 8;
+  const int slot = slot_map[t];
+  // this thread's first eight columns are asked for before the angles are made: their way from memory
+  // is then hidden behind the sines and cosines (and the barrier after them)
+  float first_v[8];
+  const bool first_live = static_cast<int>(threadIdx.x) < heads * per_head;
+  if (first_live)
+    load8(qkv + (static_cast<size_t>(t) * heads + threadIdx.x / per_head) * d + (threadIdx.x % per_head) * 8, first_v);
   if (inv_freq != nullptr) {
     const float pos = static_cast<float>(positions[t]);
     for (int i = threadIdx.x; i < half; i += blockDim.x) sincosf(pos * inv_freq[i], &sines[i], &cosines[i]);
     __syncthreads();
   }
-  const int heads = nq + 2 * nkv, per_head = d / 8;
-  const int slot = slot_map[t];
   const size_t head_stride = static_cast<size_t>(page_size) * d;
   A* page = cache + static_cast<size_t>(slot < 0 ? 0 : slot / page_size) * 2 * nkv * head_stride;
   const int row = slot < 0 ? 0 : slot % page_size;
@@ -101,7 +107,12 @@ __global__ void rope_cache_wide_kernel(const D* __restrict__ qkv, const int* __r
     const int head = g / per_head, c = (g % per_head) * 8;
     if (head >= nq && slot < 0) continue;
     float v[8];
-    load8(qkv + (static_cast<size_t>(t) * heads + head) * d + c, v);
+    if (g == static_cast<int>(threadIdx.x)) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = first_v[j];
+    } else {
+      load8(qkv + (static_cast<size_t>(t) * heads + head) * d + c, v);
+    }
     if (head >= nq + nkv) {
       // a value head: after the nkv key heads of the page, transposed
       A* out = page + (head - nq) * head_stride + static_cast<size_t>(c) * page_size + row;

@@ -104,9 +104,18 @@ class Scheduled:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_tokens_per_step: int = 2048, max_seqs_per_step: int = 64,
-                 chunk_size: int | None = None, max_positions: int | None = None, eos_token_id: int = -1):
+                 chunk_size: int | None = None, max_positions: int | None = None, eos_token_id: int = -1,
+                 prompt_tokens_beside_decodes: int | None = None):
+        """prompt_tokens_beside_decodes: in a step that holds decoding requests, prompts get at most
+        this many tokens in all (None: whatever the budget leaves).  A step's time grows with its
+        prompt tokens, and every decoding request of the step waits for it: the cap trades the
+        prompts' throughput for the decoding requests' time between tokens (the reference's steps
+        hold one token per row, prompt rows too: app/server.cpp:389-408,432-444)."""
         if max_tokens_per_step < 1 or max_seqs_per_step < 1:
             raise invalid_argument("the step budgets must be positive")
+        if prompt_tokens_beside_decodes is not None and prompt_tokens_beside_decodes < 1:
+            raise invalid_argument("prompts need at least one token a step beside decoding requests")
+        self.prompt_tokens_beside_decodes = prompt_tokens_beside_decodes
         self.cache = cache
         self.max_tokens_per_step = max_tokens_per_step
         self.max_seqs_per_step = max_seqs_per_step
@@ -201,6 +210,9 @@ class Scheduler:
                 planned.discard(victim.id)
             if request.state == "running":
                 take(request, 1, needed)
+
+        if plan and self.prompt_tokens_beside_decodes is not None:
+            budget = min(budget, self.prompt_tokens_beside_decodes)    # the decoding requests wait for the whole step
 
         # 2. running requests still in their prompt (or being recomputed), in admission order
         for request in sorted(self.running, key=lambda candidate: candidate.order):

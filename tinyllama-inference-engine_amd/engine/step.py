@@ -62,7 +62,10 @@ class StepContext:
     (those from index seq_start[num_seqs] on) are token 0 at position 0, belong to no request
     (`token_slot` -1), are written nowhere (slot maps -1) and their results are dropped; padding
     sequences have `seq_slot` -1 and, in a step of portions, no tokens.  A part that keeps state
-    per request must change it only for tokens and sequences whose slot is not negative."""
+    per request must change it only for tokens and sequences whose slot is not negative, and must
+    not let a padding token's activations reach a live token's: they may hold anything (a kernel
+    may leave the rows of tokens that belong to no sequence unwritten), also values that are not
+    finite, so they are selected away, not multiplied by zero."""
     num_tokens: int
     num_seqs: int
     num_wanted: int

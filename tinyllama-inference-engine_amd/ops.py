@@ -660,6 +660,11 @@ def attention_plan(ctx, groups_per_kv: int, num_kv_heads: int, head_dim: int):
         while (waves * 2 <= attention_max_waves(head_dim) and tiles_all * nsplit * waves * 2 <= 2048
                and ctx.max_context >= nsplit * waves * 2 * 128):
             waves *= 2
+        if nsplit > 1 and ctx.max_context <= 256 and attention_max_waves(head_dim) >= 2:
+            # up to 256 positions there is nothing to cut: two waves of one workgroup share the keys and the
+            # merge launch goes (batch 1 at 200 positions 0.902 ms a step against 0.919, batch 8 0.998
+            # against 1.017; at 450 positions the parts win again: 0.928 against 0.944 with 1 x 4)
+            nsplit, waves = 1, 2
     if nsplit == 1:
         return tiles, col_tiles, 1, 0, waves, shared
     split_len = ((ctx.max_context + nsplit - 1) // nsplit + 31) // 32 * 32

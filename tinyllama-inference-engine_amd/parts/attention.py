@@ -75,8 +75,11 @@ class Attention(Mixer):
 
     @property
     def graph_safe(self) -> bool:
-        # a position encoding applied as tensors may do anything; a rotation table (or none) is fused
-        return self.position.rotary_table() is not None or type(self.position).apply_qk is PositionEncoding.apply_qk
+        # a rotation table (or none) is fused into this part's own kernels; a position encoding applied
+        # as tensors (`apply_qk`) may do anything, so it says itself whether its launches may be recorded
+        if self.position.rotary_table() is not None or type(self.position).apply_qk is PositionEncoding.apply_qk:
+            return True
+        return bool(getattr(self.position, "graph_safe", False))
 
     adds_to_residual = True
 
