@@ -419,7 +419,7 @@ def test_gemm_skinny_launch_shapes(rows):
     first = ops.gemm_skinny(x, w, b, split_len=320, waves=4, strips=1)
     assert first.nsplit == 3
     assert rel_err(first.dense().cpu(), plain_linear(x.cpu().double(), w.cpu().double(), b.cpu().double())) < 5e-6
-    for waves in range(4, 17):
+    for waves in range(3, 17):
         for strips in (1, 2):
             if strips == 2 and (rows <= 32 or waves > 8):
                 with pytest.raises(ops.EngineError):
@@ -431,9 +431,23 @@ def test_gemm_skinny_launch_shapes(rows):
     planned = ops.gemm_skinny(x, w, b)
     assert planned.nsplit == (k + split_len - 1) // split_len and 4 <= waves <= 16 and strips in (1, 2)
     assert rel_err(planned.dense().cpu(), plain_linear(x.cpu().double(), w.cpu().double(), b.cpu().double())) < 5e-6
-    for bad in (dict(waves=3), dict(waves=17), dict(strips=3)):
+    for bad in (dict(waves=2), dict(waves=17), dict(strips=3)):
         with pytest.raises(ops.EngineError):
             ops.gemm_skinny(x, w, b, split_len=320, **{"waves": 4, "strips": 1, **bad})
+    # the gated form: all of K in a workgroup, silu(gate) * up stored by the product itself, for every launch shape
+    # (W's rows alternate gate and up), against the plain activation of the plain product
+    y = plain_linear(x.cpu().double(), w.cpu().double(), b.cpu().double())
+    want = plain_silu_mul(y[:, 0::2], y[:, 1::2])
+    for waves, strips in ((3, 1), (4, 1), (7, 1), (16, 1), (5, 2), (8, 2), (None, None)):
+        if strips == 2 and rows <= 32:
+            continue
+        got = ops.gemm_skinny(x, w, b, waves=waves, strips=strips, gated=True)
+        assert got.dtype == torch.bfloat16 and got.shape == (rows, n // 2)
+        assert rel_err(got.cpu(), want) < 6e-3, (waves, strips)                  # one rounding to bfloat16
+    with pytest.raises(ops.EngineError):
+        ops.gemm_skinny(x, w, b, split_len=320, gated=True)                      # the gated product does not split K
+    with pytest.raises(ops.EngineError):
+        ops.gemm_skinny(x, w[:999].contiguous(), b[:999].contiguous(), gated=True)   # an odd number of rows: a gate without its up
 
 
 @pytest.mark.parametrize("shape", [(15832, 2560, 2048), (40000, 2048, 5632), (70000, 704, 512), (65, 96, 64), (300, 32000, 256)])

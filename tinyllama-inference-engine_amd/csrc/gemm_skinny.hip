@@ -36,10 +36,13 @@ constexpr int kSkinnyPad = 8;                // bf16 elements of padding per LDS
 // the unit with the most bytes; 176 workgroups on 256 units measured 3.1 TB/s, 256 of them 4.3).
 // CHUNK: k values staged in LDS at a time.
 // split_len: k values per split (multiple of 64).  K % 8 == 0.
-template <int NT, int RS, int CHUNK, int MINWAVES, int MAXWAVES>
+// GATED: K is not split (one split holds all of it), W's rows alternate gate and up (g0, u0, g1, u1, ...),
+// and the workgroup, which then holds complete sums, stores silu(gate) * up as bfloat16 [M, N / 2] in `act`
+// instead of partial sums: the activation kernel's launch, and the partial sums' way to memory and back, go.
+template <int NT, int RS, int CHUNK, int MINWAVES, int MAXWAVES, bool GATED = false>
 __global__ void __launch_bounds__(64 * MAXWAVES)
 gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ w, const uint16_t* __restrict__ bias,
-                   float* __restrict__ y, int M, int N, int K, int split_len) {
+                   float* __restrict__ y, uint16_t* __restrict__ act, int M, int N, int K, int split_len) {
   constexpr int kStride = CHUNK + kSkinnyPad;
   constexpr int kSteps = CHUNK / 64;
   __shared__ __attribute__((aligned(16))) uint16_t xs[NT * 16 * kStride];
@@ -148,6 +151,16 @@ gemm_skinny_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ 
     for (int t = 0; t < NT; ++t) {
       const int token = t * 16 + (lane & 15);
       if (token >= M) continue;
+      if (GATED) {
+        // (N is even and n0 a multiple of 4: a gate and its up are neighbours in this lane)
+        const float g0 = acc[r][t][0] + add[0], u0 = acc[r][t][1] + add[1], g1 = acc[r][t][2] + add[2], u1 = acc[r][t][3] + add[3];
+        uint16_t* gated = act + static_cast<size_t>(token) * (N / 2) + (n0 >> 1);
+        if (n0 + 3 < N)
+          *reinterpret_cast<uint32_t*>(gated) = pack_bf16((g0 / (1.f + expf(-g0))) * u0, (g1 / (1.f + expf(-g1))) * u1);
+        else if (n0 + 1 < N)
+          gated[0] = __bfloat16_as_ushort(__float2bfloat16((g0 / (1.f + expf(-g0))) * u0));
+        continue;
+      }
       float* out = y + (static_cast<size_t>(split) * M + token) * N + n0;
       if ((N & 3) == 0 && n0 + 3 < N) {
         *reinterpret_cast<float4*>(out) =
@@ -167,37 +180,52 @@ using namespace tlie;
 
 namespace {
 
-template <int NT, int RS>
-int launch_skinny(dim3 grid, int waves, hipStream_t s, const uint16_t* x, const uint16_t* w, const uint16_t* bias, float* y, int M,
-                  int N, int K, int split_len) {
+template <int NT, int RS, bool GATED>
+int launch_skinny(dim3 grid, int waves, hipStream_t s, const uint16_t* x, const uint16_t* w, const uint16_t* bias, float* y,
+                  uint16_t* act, int M, int N, int K, int split_len) {
   // (the staged chunk is as long as the registers allow for the workgroup's size)
   const dim3 block(64 * waves);
-  if (waves <= 4) {
+  if (waves == 3) {
     constexpr int kChunk = NT <= 2 ? 512 : 256;
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 4, 4>), grid, block, 0, s, x, w, bias, y, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 3, 3, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
+  } else if (waves <= 4) {
+    constexpr int kChunk = NT <= 2 ? 512 : 256;
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 4, 4, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
   } else if (waves <= 8) {
     constexpr int kChunk = RS == 1 ? 256 : 128;
-    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 5, 8>), grid, block, 0, s, x, w, bias, y, M, N, K, split_len);
+    hipLaunchKernelGGL((gemm_skinny_kernel<NT, RS, kChunk, 5, 8, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
   } else {
     if constexpr (RS == 1)
-      hipLaunchKernelGGL((gemm_skinny_kernel<NT, 1, (NT <= 2 ? 256 : 128), 9, 16>), grid, block, 0, s, x, w, bias, y, M, N, K, split_len);
+      hipLaunchKernelGGL((gemm_skinny_kernel<NT, 1, (NT <= 2 ? 256 : 128), 9, 16, GATED>), grid, block, 0, s, x, w, bias, y, act, M, N, K, split_len);
     else
       return kBadArgument;
   }
   return launch_status();
 }
 
+template <bool GATED>
+int dispatch_skinny(dim3 grid, int waves, int strips, int tiles, hipStream_t s, const uint16_t* x, const uint16_t* w,
+                    const uint16_t* bias, float* y, uint16_t* act, int M, int N, int K, int split_len) {
+  if (tiles <= 1) return launch_skinny<1, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
+  if (tiles == 2) return launch_skinny<2, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
+  if (strips == 1) return launch_skinny<4, 1, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
+  return launch_skinny<4, 2, GATED>(grid, waves, s, x, w, bias, y, act, M, N, K, split_len);
+}
+
 }  // namespace
 
 // x [M, K], w [N, K], bias [N] or null: bfloat16.  y: float [nsplit, M, N] with
 // nsplit = ceil(K / split_len).  M <= 64, K % 8 == 0, split_len % 64 == 0.
-// waves: 4 to 16 waves a workgroup; strips: 1 or 2 strips of 16 rows of W per wave (2 only for more
+// waves: 3 to 16 waves a workgroup; strips: 1 or 2 strips of 16 rows of W per wave (2 only for more
 // than 32 rows of x and up to 8 waves); a workgroup takes 16 * strips * waves rows of W.
-extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, float* y, int M, int N, int K,
+// act (or null): with it, split_len must cover K (one split), N must be even, W's rows alternate gate and up, and
+// bfloat16 silu(gate) * up [M, N / 2] is stored there instead of y (which may then be null).
+extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, float* y, void* act, int M, int N, int K,
                                 int split_len, int waves, int strips, void* stream) {
   if (M <= 0 || M > 64 || N <= 0 || K <= 0 || (K & 7) != 0 || split_len <= 0 || (split_len & 63) != 0) return kBadArgument;
-  if (waves < 4 || waves > 16 || strips < 1 || strips > 2 || (strips == 2 && (M <= 32 || waves > 8))) return kBadArgument;
+  if (waves < 3 || waves > 16 || strips < 1 || strips > 2 || (strips == 2 && (M <= 32 || waves > 8))) return kBadArgument;
   const int nsplit = (K + split_len - 1) / split_len;
+  if (act != nullptr ? (nsplit != 1 || (N & 1) != 0) : y == nullptr) return kBadArgument;
   const int tiles = (M + 15) / 16;
   const int rows_per_block = 16 * strips * waves;
   const dim3 grid((N + rows_per_block - 1) / rows_per_block, nsplit);
@@ -206,8 +234,6 @@ extern "C" int tlie_gemm_skinny(const void* x, const void* w, const void* bias, 
   const uint16_t* xp = (const uint16_t*)x;
   const uint16_t* wp = (const uint16_t*)w;
   const uint16_t* bp = (const uint16_t*)bias;
-  if (tiles <= 1) return launch_skinny<1, 1>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
-  if (tiles == 2) return launch_skinny<2, 1>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
-  if (strips == 1) return launch_skinny<4, 1>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
-  return launch_skinny<4, 2>(grid, waves, s, xp, wp, bp, y, M, N, K, split_len);
+  if (act != nullptr) return dispatch_skinny<true>(grid, waves, strips, tiles, s, xp, wp, bp, y, (uint16_t*)act, M, N, K, split_len);
+  return dispatch_skinny<false>(grid, waves, strips, tiles, s, xp, wp, bp, y, nullptr, M, N, K, split_len);
 }

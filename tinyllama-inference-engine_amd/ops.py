@@ -519,10 +519,27 @@ def gemm_skinny_takes(x: torch.Tensor, weight: torch.Tensor) -> bool:
             and weight.shape[1] % 8 == 0)
 
 
+def skinny_gated_plan(rows: int, out_features: int, in_features: int, compute_units: int = 256) -> tuple[int, int]:
+    """(waves a workgroup, strips a wave) of `gemm_skinny` when it keeps all of K in a workgroup and applies
+    the SiLU gate itself: as many equal workgroups as compute units, or just fewer (see `skinny_plan`); a
+    workgroup's time is its rows of W from memory and all of x from the caches."""
+    best = None
+    for strips in ((1, 2) if rows > 32 else (1,)):
+        for waves in range(3, (8 if strips == 2 else 16) + 1):
+            blocks = -(-out_features // (16 * waves * strips))
+            rounds = -(-blocks // compute_units)
+            cost = rounds * (16 * waves * strips * in_features * 2 / 20e3 + 0.5)
+            if best is None or cost < best[0]:
+                best = (cost, waves, strips)
+    return best[1], best[2]
+
+
 def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, split_len: int | None = None,
-                waves: int | None = None, strips: int | None = None) -> Product:
+                waves: int | None = None, strips: int | None = None, gated: bool = False):
     """y = x . W^T (+ bias) for at most 64 rows of bfloat16 x: float partial sums [nsplit, M, N].
-    split_len, waves, strips: the launch shape (see `skinny_plan`, which chooses it when they are not given)."""
+    split_len, waves, strips: the launch shape (see `skinny_plan`, which chooses it when they are not given).
+    gated: W's rows alternate gate and up; K is not split, and the kernel stores bfloat16
+    silu(gate) * up [M, N / 2], which is returned as a tensor (no partial sums, no activation kernel)."""
     _device_tensor(x, "x", torch.bfloat16)
     _device_tensor(weight, "weight", torch.bfloat16)
     if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -534,17 +551,30 @@ def gemm_skinny(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None
         _device_tensor(bias, "bias", torch.bfloat16)
         if bias.shape != (out_features,):
             raise invalid_shape("gemm_skinny: bias needs one entry per output")
-    if split_len is None:
+    if gated:
+        if out_features % 2 != 0:
+            raise invalid_shape("gemm_skinny: the gated product needs an even number of rows of W")
+        if split_len is not None and split_len < in_features:
+            raise invalid_argument("gemm_skinny: the gated product does not split K")
+        split_len = (in_features + 63) // 64 * 64
+        if waves is None or strips is None:
+            waves, strips = skinny_gated_plan(rows, out_features, in_features, _compute_units(x.device))
+    elif split_len is None:
         split_len, waves, strips = skinny_plan(rows, out_features, in_features, _compute_units(x.device))
     elif waves is None or strips is None:
         waves, strips = waves or 4, strips or (2 if rows > 32 else 1)
     if split_len <= 0 or split_len % 64 != 0:
         raise invalid_argument("gemm_skinny: a split's length must be a positive multiple of 64")
-    if not 4 <= waves <= 16 or strips not in (1, 2) or (strips == 2 and (rows <= 32 or waves > 8)):
-        raise invalid_argument("gemm_skinny: 4 to 16 waves; two strips a wave only for more than 32 rows and up to 8 waves")
+    if not 3 <= waves <= 16 or strips not in (1, 2) or (strips == 2 and (rows <= 32 or waves > 8)):
+        raise invalid_argument("gemm_skinny: 3 to 16 waves; two strips a wave only for more than 32 rows and up to 8 waves")
     nsplit = (in_features + split_len - 1) // split_len
+    if gated:
+        act = torch.empty((rows, out_features // 2), dtype=torch.bfloat16, device=x.device)
+        _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(None), _ptr(act), rows, out_features, in_features,
+                                          split_len, waves, strips, _stream()), "gemm_skinny")
+        return act
     out = torch.empty((nsplit, rows, out_features), dtype=torch.float32, device=x.device)
-    _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), rows, out_features, in_features,
+    _check(library().tlie_gemm_skinny(_ptr(x), _ptr(weight), _ptr(bias), _ptr(out), _ptr(None), rows, out_features, in_features,
                                       split_len, waves, strips, _stream()), "gemm_skinny")
     return Product(out, nsplit)
 

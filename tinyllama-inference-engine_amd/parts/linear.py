@@ -6,7 +6,8 @@ Which kernel runs is decided here and nowhere else:
   bfloat16, weight kept float32  the same kernel on widened values
   bfloat16, at most 16 rows      the rows kernel when the caller folds something in: the norm before the
                                  product, the SiLU gate or the add into the residual after it
-  bfloat16, at most 64 rows      the skinny MFMA kernel (W streamed once, split-K partial sums)
+  bfloat16, at most 64 rows      the skinny MFMA kernel (W streamed once, split-K partial sums; the gated
+                                 feed-forward's first product keeps K whole and applies the SiLU gate itself)
   bfloat16, more rows            the library's product (as the reference uses a library for its
                                  products: cublasGemmEx, src/cuda/kernels.cu:342-368), bfloat16 out, or
                                  float32 for the output head: hipBLASLt called directly
@@ -58,6 +59,8 @@ class Linear:
                 return ops.gemm_rows(x, self.weight, self.bias, "store")
         if isinstance(x, ops.NormedRows):
             raise ops.invalid_argument("this product cannot fold the norm before it; ask takes_rows() first")
+        if gated and ops.gemm_skinny_takes(x, self.weight) and self.out_features % 2 == 0:
+            return ops.gemm_skinny(x, self.weight, self.bias, gated=True)     # all of K in a workgroup: the gate is applied there
         if ops.gemm_skinny_takes(x, self.weight) and (not whole or out_dtype == torch.float32):
             split_len = (self.in_features + 63) // 64 * 64 if whole else None
             return ops.gemm_skinny(x, self.weight, self.bias, split_len=split_len)
