@@ -122,7 +122,9 @@ def bench_kernels(cfg: dict, batch: int = 8, context: int = 2048, prompt: int = 
             count = _copies(n * k * 2)
             weights = [rand(n, k) for _ in range(count)]
             x = rand(batch, k, scale=1.0)
-            if batch <= ops.SKINNY_MAX_ROWS:
+            if batch <= ops.SKINNY_MAX_ROWS and name == "gate_up":
+                launch, kind = (lambda i: ops.gemm_skinny(x, weights[i], None, gated=True)), "gemm_skinny (gated)"
+            elif batch <= ops.SKINNY_MAX_ROWS:
                 launch, kind = (lambda i: ops.gemm_skinny(x, weights[i], None)), "gemm_skinny"
             else:
                 launch, kind = (lambda i: ops.library_mm(x, weights[i], torch.float32 if name == "head" else bf)), "library"
