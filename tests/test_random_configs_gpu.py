@@ -59,9 +59,10 @@ def weight_std(hidden):
 
 
 # How far below the plain logits' best a bfloat16 engine's greedy token may lie, as a share of the
-# row's largest logit: the engine's logits are within 1.5e-2 of the plain ones row by row
-# (gpu_helpers.TOLERANCE), so a token it prefers is within twice that of the best.
-BF16_TOKEN_GAP = 3e-2
+# row's largest logit.  Measured over these 40 draws: 0 in all but two, 3.7e-3 at the most (width 1920,
+# three layers); the bound leaves that room and no more (the engine's logits may be 1.5e-2 from the
+# plain ones row by row, gpu_helpers.TOLERANCE, but a greedy token turns only at a near tie).
+BF16_TOKEN_GAP = 1e-2
 
 
 def run_case(tmp_path, seed, wide):
@@ -90,7 +91,8 @@ def run_case(tmp_path, seed, wide):
 
 @pytest.mark.parametrize("seed", range(24))
 def test_random_configuration_and_workload(tmp_path, seed):
-    run_case(tmp_path, seed, wide=False)
+    case, worst = run_case(tmp_path, seed, wide=False)
+    print(f"seed {seed} {case['dtype']} width {case['config']['hidden_size']}: a token lies at most {worst:.2e} of its row's scale below the best")
 
 
 @pytest.mark.parametrize("seed", range(100, 116))
