@@ -1047,3 +1047,36 @@ def test_pool_sized_by_a_share_of_free_memory_and_byte_budgets(setups):
         assert caught.value.code == ErrorCode.OUT_OF_MEMORY and "budget" in caught.value.message
     with pytest.raises(EngineError):
         Engine(setup["folder"], dtype="bfloat16", max_tokens=None)
+
+
+def test_the_weights_lie_in_one_allocation_and_load_part_by_part(tmp_path):
+    """What the parts keep lies in the engine's one weight allocation, each tensor at a multiple of 256
+    bytes, a tied head on the table's place; and while a model loads, the device never holds much more than
+    that allocation: stored tensors come when a part asks and go when it has loaded (a load that brought
+    all stored tensors first would hold twice the weights at its peak)."""
+    from tlie_amd import Engine
+    raw = dict(CONFIGS["A"], hidden_size=512, intermediate_size=1024, num_hidden_layers=12, num_attention_heads=8,
+               num_key_value_heads=2, head_dim=64, vocab_size=1000, tie_word_embeddings=True)
+    folder = make_model(tmp_path / "model", raw, seed=4, dtype_name="bfloat16", std=0.02)
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    engine = Engine(folder, dtype="bfloat16", max_tokens=64, page_size=16, max_requests=2)
+    peak = torch.cuda.max_memory_allocated() - before
+    arena = engine.weight_arena
+    model = engine.model
+    kept = [model.embedding.table, model.final_norm.weight, model.head.linear.weight]
+    for block in model.blocks:
+        kept += [block.mixer.qkv.weight, block.mixer.o.weight, block.feed_forward.gate_up.weight, block.feed_forward.down.weight,
+                 block.mixer_norm.weight, block.feed_forward_norm.weight]
+    assert all(arena.holds(tensor) and tensor.data_ptr() % 256 == 0 for tensor in kept) and arena.outside == 0
+    assert model.head.linear.weight.data_ptr() == model.embedding.table.data_ptr()
+    stored = os.path.getsize(os.path.join(folder, "model.safetensors"))
+    assert 0.98 * stored < arena.used <= arena.capacity < 1.02 * stored
+    assert peak < 1.4 * arena.capacity, (peak, arena.capacity)
+    tokens = random_tokens(3, 20, 1000)
+    plain = plain_forward(*load_plain(folder), tokens)
+    replay = Replayer(engine)
+    replay.step([("r", tokens, list(range(20)))], end=["r"])
+    assert_close(replay.logits_of("r", range(20)), plain, TOLERANCE["bfloat16"], "a model in the arena, whole")

@@ -203,3 +203,72 @@ def test_a_byte_budget_refuses_the_weight_files_before_mapping(tmp_path):
     WeightStore(str(tmp_path), max_file_bytes=size).validate(specs)
     error = code_of(lambda: WeightStore(str(tmp_path), max_file_bytes=size - 1))
     assert error.code == ErrorCode.OUT_OF_MEMORY and "budget" in error.message
+
+
+def test_the_arena_hands_out_aligned_places_and_says_when_it_is_full():
+    from tlie_amd.weights import WeightArena
+    arena = WeightArena(1000, "cpu")
+    assert arena.capacity == 1024
+    a = arena.place(torch.arange(10, dtype=torch.float32))                  # 40 bytes: one place of 256
+    b = arena.place(torch.arange(190, dtype=torch.int32).view(10, 19))      # 760 bytes: three more, the arena is full
+    assert a.data_ptr() % 256 == 0 and b.data_ptr() == a.data_ptr() + 256 and arena.used == 1024
+    assert torch.equal(a, torch.arange(10, dtype=torch.float32)) and torch.equal(b, torch.arange(190, dtype=torch.int32).view(10, 19))
+    assert arena.holds(a) and arena.holds(b[3:]) and arena.place(b) is b and arena.used == 1024
+    late = torch.ones(3)
+    assert arena.place(late) is late and not arena.holds(late) and arena.outside == 12     # it stays where it is, and is counted
+
+
+def test_resident_weights_bring_a_tensor_when_asked_and_remember_what_was_kept_whole():
+    from tlie_amd.weights import ResidentWeights, keep_in
+    calls = []
+
+    def make(name, values):
+        def fetch():
+            calls.append(name)
+            return torch.tensor(values, dtype=torch.float32)
+        return fetch
+    weights = ResidentWeights({"a": make("a", [1.0, 2.0]), "b": make("b", [3.0]), "c": make("c", [4.0, 5.0, 6.0])},
+                              {"a": 8, "b": 4, "c": 12}, "cpu")
+    assert weights.arena.capacity == 3 * 256 and set(weights) == {"a", "b", "c"} and "a" in weights and "z" not in weights
+    assert calls == []                                                     # nothing is brought before it is asked for
+    assert weights["a"] is weights["a"] and calls == ["a"]                 # and once while the part loads
+    fused = weights.keep(torch.cat([weights["a"], weights["b"]]))          # a part fuses two and keeps the result
+    assert weights.arena.holds(fused) and fused.tolist() == [1.0, 2.0, 3.0]
+    whole = weights.keep(weights["c"])                                     # another keeps one as it came
+    weights.release()
+    assert weights["c"] is whole and calls == ["a", "b", "c"]              # that one is known by its name from then on
+    assert weights["a"].tolist() == [1.0, 2.0] and calls == ["a", "b", "c", "a"]      # a fused one is brought again
+    assert weights.get("z") is None and code_of(lambda: weights["z"]).code == ErrorCode.INVALID_SHAPE
+    plain = {"a": torch.ones(2)}
+    assert keep_in(plain, plain["a"]) is plain["a"] and keep_in(weights, whole) is whole
+
+
+def test_a_model_loaded_through_resident_weights_lies_in_one_allocation(tmp_path):
+    """On the CPU (loading launches no kernel): every matrix and norm weight of the model has its place
+    in the arena, a tied head shares the table's, each stored tensor is read once, and the values are
+    those of a model loaded from a dict."""
+    from tlie_amd.models import build_model
+    raw = dict(TINY, tie_word_embeddings=True, attention_bias=True)
+    config = LlamaConfig.from_dict(raw)
+    write_random_model(str(tmp_path), config, seed=9)
+    spec = config.to_spec()
+    store = WeightStore(str(tmp_path))
+    reads = []
+    get = store.get
+    store.get = lambda name: (reads.append(name), get(name))[1]
+    weights = store.resident(expected_tensors(spec), torch.bfloat16, "cpu")
+    model = build_model(spec, weights, torch.bfloat16, "cpu")
+    arena = weights.arena
+    kept = [model.embedding.table, model.final_norm.weight, model.head.linear.weight]
+    for block in model.blocks:
+        kept += [block.mixer.qkv.weight, block.mixer.qkv.bias, block.mixer.o.weight, block.mixer.o.bias,
+                 block.feed_forward.gate_up.weight, block.feed_forward.down.weight, block.mixer_norm.weight, block.feed_forward_norm.weight]
+    assert all(arena.holds(tensor) and tensor.data_ptr() % 256 == 0 for tensor in kept) and arena.outside == 0
+    assert model.head.linear.weight.data_ptr() == model.embedding.table.data_ptr()
+    assert sorted(reads) == sorted(spec.name for spec in expected_tensors(spec) if not spec.optional)     # each once
+    assert arena.used <= arena.capacity and not weights._fresh
+    eager = build_model(spec, WeightStore(str(tmp_path)).load(expected_tensors(spec), torch.bfloat16, "cpu"), torch.bfloat16, "cpu")
+    for mine, theirs in zip(model.blocks, eager.blocks):
+        assert torch.equal(mine.mixer.qkv.weight, theirs.mixer.qkv.weight) and torch.equal(mine.feed_forward.gate_up.weight, theirs.feed_forward.gate_up.weight)
+        assert torch.equal(mine.mixer.qkv.bias, theirs.mixer.qkv.bias) and torch.equal(mine.feed_forward.down.weight, theirs.feed_forward.down.weight)
+    assert torch.equal(model.embedding.table, eager.embedding.table)

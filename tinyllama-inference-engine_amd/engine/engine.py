@@ -65,17 +65,18 @@ class Engine:
             if expect_sha256 is not None:
                 store.expect_sha256(expect_sha256)
             with device_memory_errors("the weights"):
-                weights = store.load(expected_tensors(self.spec), self.dtype, self.device, self.spec.ignored_tensors)
+                weights = store.resident(expected_tensors(self.spec), self.dtype, self.device, self.spec.ignored_tensors)
         else:
             if config is None or random_seed is None:
                 raise invalid_argument("without a model folder the engine needs a config and a random seed")
-            from ..weights.random_init import random_tensors
+            from ..weights.random_init import resident_random_tensors
             self.config = config_from_dict(config)
             self.spec = self.config.to_spec()
             with device_memory_errors("the weights"):
-                weights = random_tensors(expected_tensors(self.spec), random_seed, dtype=self.dtype, device=self.device)
+                weights = resident_random_tensors(expected_tensors(self.spec), random_seed, dtype=self.dtype, device=self.device)
         with device_memory_errors("the weights"):
             self.model = build_model(self.spec, weights, self.dtype, self.device)
+        self.weight_arena = weights.arena                  # the one allocation that holds what the parts kept
         needs = self.model.run_needs()
         if max_tokens is None:
             if cache_fraction is None or not 0.0 < cache_fraction <= 1.0:

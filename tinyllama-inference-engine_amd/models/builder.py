@@ -40,12 +40,18 @@ class DecoderModel:
         self.final_norm = lookup("norm", spec.final_norm.kind)(spec.final_norm, dtype, device)
         self.head = lookup("head", spec.head.kind)(spec.head, dtype, device)
 
-    def load(self, weights: dict[str, torch.Tensor]) -> None:
+    def load(self, weights) -> None:
+        """weights: tensors on the device by name: a dict, or a `ResidentWeights`, which brings a
+        tensor when a part asks for it and is told after each part that what it brought may go."""
+        release = getattr(weights, "release", lambda: None)
         self.embedding.load(weights, self.spec.embedding_name)
+        release()
         for block in self.blocks:
             block.load(weights)
+            release()
         self.final_norm.load(weights, self.spec.final_norm_prefix)
         self.head.load(weights, self.spec.head_name)
+        release()
 
     @property
     def graph_safe(self) -> bool:
@@ -106,7 +112,7 @@ class DecoderModel:
         return logits
 
 
-def build_model(spec: ModelSpec, weights: dict[str, torch.Tensor], dtype: torch.dtype, device) -> DecoderModel:
+def build_model(spec: ModelSpec, weights, dtype: torch.dtype, device) -> DecoderModel:
     model = DecoderModel(spec, dtype, device)
     model.load(weights)
     return model

@@ -10,6 +10,7 @@ and the cache write are one kernel, and all tokens of a step run together.
 from __future__ import annotations
 
 import math
+from functools import partial
 
 import torch
 
@@ -17,6 +18,7 @@ from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..errors import invalid_config
 from ..registry import lookup, register
+from ..weights.arena import keep_in
 from .base import Binding, CacheNeed, Mixer, PositionEncoding
 from .linear import Linear
 
@@ -69,9 +71,10 @@ class Attention(Mixer):
         def cat(suffix):
             joined = torch.cat([weights[f"{prefix}{name}_proj.{suffix}"] for name in "qkv"], dim=0)
             return joined[order].contiguous() if order is not None else joined
-        self.qkv = Linear(cat("weight"), cat("bias") if self.bias else None, self.dtype)
+        keep = partial(keep_in, weights)
+        self.qkv = Linear(cat("weight"), cat("bias") if self.bias else None, self.dtype, keep=keep)
         self.o = Linear(weights[prefix + "o_proj.weight"], weights.get(prefix + "o_proj.bias") if self.bias else None,
-                        self.dtype)
+                        self.dtype, keep=keep)
 
     @property
     def graph_safe(self) -> bool:

@@ -6,11 +6,14 @@ product of the final norm's output with `lm_head.weight`, no bias, no scaling
 Logits are float32 whatever the activation type."""
 from __future__ import annotations
 
+from functools import partial
+
 import torch
 
 from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..registry import register
+from ..weights.arena import keep_in
 from .base import Part
 from .linear import Linear
 
@@ -31,7 +34,7 @@ class TokenEmbedding(Part):
         return [TensorSpec(name or cls.NAME, (int(spec["vocab_size"]), int(spec["hidden_size"])))]
 
     def load(self, weights, name=""):
-        self.table = weights[name or self.NAME].contiguous()
+        self.table = keep_in(weights, weights[name or self.NAME].contiguous())
 
     def forward(self, tokens: torch.Tensor, ctx=None) -> torch.Tensor:
         """The float32 residual [T, H] of the step's tokens.  `ctx` is the step's context: an
@@ -64,7 +67,7 @@ class LMHead(Part):
 
     def load(self, weights, name=""):
         matrix = weights[self.tied_to] if self.tied else weights[name or self.NAME]
-        self.linear = Linear(matrix, None, self.dtype)
+        self.linear = Linear(matrix, None, self.dtype, keep=partial(keep_in, weights))
 
     def takes_normed_rows(self, rows: int) -> bool:
         return self.linear.takes_rows(rows)

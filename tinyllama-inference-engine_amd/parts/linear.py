@@ -23,11 +23,14 @@ from ..ops import Product
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None, dtype: torch.dtype):
-        self.weight = weight.contiguous()
-        self.bias = bias.contiguous() if bias is not None else None
-        if self.bias is not None and self.bias.dtype != self.weight.dtype:
-            self.bias = self.bias.to(self.weight.dtype)
+    def __init__(self, weight: torch.Tensor, bias: torch.Tensor | None, dtype: torch.dtype, keep=None):
+        """keep: what gives a tensor its place for good (`keep_in` of the mapping that the part loads
+        from); without it the tensors stay where they are."""
+        keep = keep or (lambda tensor: tensor)
+        self.weight = keep(weight.contiguous())
+        if bias is not None and bias.dtype != self.weight.dtype:
+            bias = bias.to(self.weight.dtype)
+        self.bias = keep(bias.contiguous()) if bias is not None else None
         self.dtype = dtype
         self.out_features, self.in_features = self.weight.shape
 

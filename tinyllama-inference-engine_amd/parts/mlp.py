@@ -4,12 +4,15 @@ weight [2 * inter, hidden] whose rows alternate gate and up (g0, u0, g1, u1, ...
 few rows then has a gate and its up in one lane and applies the activation itself."""
 from __future__ import annotations
 
+from functools import partial
+
 import torch
 
 from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..errors import invalid_config
 from ..registry import register
+from ..weights.arena import keep_in
 from .base import FeedForward
 from .linear import Linear
 
@@ -37,8 +40,9 @@ class GatedMLP(FeedForward):
 
     def load(self, weights, prefix):
         gate, up = weights[prefix + "gate_proj.weight"], weights[prefix + "up_proj.weight"]
-        self.gate_up = Linear(torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden), None, self.dtype)
-        self.down = Linear(weights[prefix + "down_proj.weight"], None, self.dtype)
+        keep = partial(keep_in, weights)
+        self.gate_up = Linear(torch.stack([gate, up], dim=1).reshape(2 * self.inter, self.hidden), None, self.dtype, keep=keep)
+        self.down = Linear(weights[prefix + "down_proj.weight"], None, self.dtype, keep=keep)
 
     adds_to_residual = True
 

@@ -8,6 +8,7 @@ import torch
 from .. import ops
 from ..config.spec import PartSpec, TensorSpec
 from ..registry import register
+from ..weights.arena import keep_in
 from .base import Norm, ResidualUpdated, as_product
 
 
@@ -27,7 +28,7 @@ class RMSNorm(Norm):
         return [TensorSpec(prefix + "weight", (int(spec["size"]),), init="norm")]
 
     def load(self, weights, prefix):
-        self.weight = weights[prefix + "weight"].contiguous()
+        self.weight = keep_in(weights, weights[prefix + "weight"].contiguous())
 
     def forward(self, residual):
         return ops.add_rmsnorm(residual, None, self.weight, self.eps, self.dtype)

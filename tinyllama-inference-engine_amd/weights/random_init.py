@@ -29,22 +29,39 @@ def random_tensors(specs: list[TensorSpec], seed: int, std: float = 0.02, norm_s
                    dtype: torch.dtype = torch.bfloat16, device="cpu") -> dict[str, torch.Tensor]:
     """Drawn on `device`; the values of a (seed, name) are the same on every run on one kind of
     device, but differ between the CPU's and the GPU's generators."""
-    out = {}
-    for spec in specs:
-        if spec.optional:
-            continue
-        generator = _generator(seed, spec.name, device)
-        values = torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device)
-        if spec.init == "normal":
-            values = values * std
-        elif spec.init == "norm":
-            values = 1.0 + values * norm_std
-        elif spec.init == "zeros":
-            values = torch.zeros(spec.shape, device=device)
-        else:
-            raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
-        out[spec.name] = values.to(dtype)
-    return out
+    return {spec.name: _draw(spec, seed, std, norm_std, dtype, device) for spec in specs if not spec.optional}
+
+
+def _draw(spec: TensorSpec, seed: int, std: float, norm_std: float, dtype: torch.dtype, device) -> torch.Tensor:
+    generator = _generator(seed, spec.name, device)
+    values = torch.randn(spec.shape, generator=generator, dtype=torch.float32, device=device)
+    if spec.init == "normal":
+        values = values * std
+    elif spec.init == "norm":
+        values = 1.0 + values * norm_std
+    elif spec.init == "zeros":
+        values = torch.zeros(spec.shape, device=device)
+    else:
+        raise ValueError(f"unknown init '{spec.init}' for {spec.name}")
+    return values.to(dtype)
+
+
+def resident_random_tensors(specs: list[TensorSpec], seed: int, std: float = 0.02, norm_std: float = 0.01,
+                            dtype: torch.dtype = torch.bfloat16, device="cpu"):
+    """The tensors of `random_tensors`, each drawn when a part asks for it, as a `ResidentWeights`
+    (one device allocation for what the parts keep)."""
+    from .arena import ResidentWeights
+    wanted = [spec for spec in specs if not spec.optional]
+
+    def draw(spec):
+        return lambda: _draw(spec, seed, std, norm_std, dtype, device)
+    sizes = {}
+    for spec in wanted:
+        count = 1
+        for extent in spec.shape:
+            count *= int(extent)
+        sizes[spec.name] = count * dtype.itemsize
+    return ResidentWeights({spec.name: draw(spec) for spec in wanted}, sizes, device)
 
 
 def write_random_model(model_dir: str, config, seed: int, std: float = 0.02, norm_std: float = 0.01,

@@ -121,36 +121,58 @@ class WeightStore:
 
     def load(self, specs: Iterable[TensorSpec], dtype: torch.dtype, device,
              ignored: Iterable[str] = ()) -> dict[str, torch.Tensor]:
-        """Validates, then uploads every required tensor, in its kept precision.  A tensor the
+        """Validates, then uploads every required tensor, in its kept precision, each an allocation
+        of its own (see `resident` for what the engine uses).  A tensor the
         model marks optional (a tied head's matrix that some files still carry) is checked when
         present and not uploaded: no part reads it.  A matrix stored in 32-bit stays 32-bit also in
         a bfloat16 run (its products then go to the true 32-bit kernel, at a fraction of the
         speed): that is said once, as a warning, because nothing else shows it."""
+        names = self._checked(specs, dtype, ignored)
+        return {name: to_kept_precision(self.get(name), dtype).to(device) for name in names}
+
+    def resident(self, specs: Iterable[TensorSpec], dtype: torch.dtype, device, ignored: Iterable[str] = ()):
+        """Validates like `load`, uploads nothing yet: a `ResidentWeights` that uploads a tensor when a
+        part asks for it, with one device allocation for everything that the parts keep."""
+        from .arena import ResidentWeights
+        names = self._checked(specs, dtype, ignored)
+
+        def upload(name):
+            return lambda: to_kept_precision(self.get(name), dtype).to(device)
+        sizes = {}
+        for name in names:
+            entry = self._where[name].tensors[name]
+            count = 1
+            for extent in entry.shape:
+                count *= int(extent)
+            sizes[name] = count * kept_dtype(entry.dtype, dtype).itemsize
+        return ResidentWeights({name: upload(name) for name in names}, sizes, device)
+
+    def _checked(self, specs: Iterable[TensorSpec], dtype: torch.dtype, ignored: Iterable[str]) -> list[str]:
+        """The names to upload, after validation and the warning about matrices stored in 32-bit."""
         specs = list(specs)
         self.validate(specs, ignored)
-        out, wide = {}, []
-        for spec in specs:
-            if spec.name in self._where and not spec.optional:
-                kept = to_kept_precision(self.get(spec.name), dtype)
-                if dtype == torch.bfloat16 and kept.dtype == torch.float32 and kept.dim() >= 2:
-                    wide.append(spec.name)
-                out[spec.name] = kept.to(device)
+        names = [spec.name for spec in specs if spec.name in self._where and not spec.optional]
+        wide = [name for name in names if dtype == torch.bfloat16 and len(self.shape(name)) >= 2
+                and kept_dtype(self._where[name].tensors[name].dtype, dtype) == torch.float32]
         if wide:
             import warnings
             warnings.warn(f"{len(wide)} matrices of {self.model_dir} are stored in 32-bit and are kept so in this bfloat16 run "
                           f"(first: {wide[0]}); their products take the 32-bit kernel, which is many times slower",
-                          stacklevel=2)
-        return out
+                          stacklevel=3)
+        return names
+
+
+def kept_dtype(stored: torch.dtype, dtype: torch.dtype) -> torch.dtype:
+    """The type a tensor stored as `stored` is kept in when the model runs in `dtype`."""
+    if stored in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool):
+        return torch.int32
+    if dtype == torch.float32:
+        return torch.float32
+    if dtype == torch.bfloat16:
+        return torch.float32 if stored in (torch.float32, torch.float64) else torch.bfloat16
+    raise EngineError(ErrorCode.INVALID_DTYPE, f"the engine runs in bfloat16 or float32, not {dtype}")
 
 
 def to_kept_precision(tensor: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
-    """The precision a stored tensor is kept in when the model runs in `dtype`."""
-    if tensor.dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool):
-        return tensor.to(torch.int32)
-    if dtype == torch.float32:
-        return tensor.to(torch.float32)
-    if dtype == torch.bfloat16:
-        if tensor.dtype in (torch.float32, torch.float64):
-            return tensor.to(torch.float32)
-        return tensor.to(torch.bfloat16)
-    raise EngineError(ErrorCode.INVALID_DTYPE, f"the engine runs in bfloat16 or float32, not {dtype}")
+    """The stored tensor in the precision it is kept in when the model runs in `dtype`."""
+    return tensor.to(kept_dtype(tensor.dtype, dtype))
