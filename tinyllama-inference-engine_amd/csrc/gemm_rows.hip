@@ -72,6 +72,71 @@ struct RowsArgs {
   uint16_t* cache;            // [pages, 2, nkv, page_size * d]: keys [row][dim], values [dim][row]
 };
 
+// S whole steps of 64 k for every strip: all of W's pieces are asked for first (16 bytes a lane and piece;
+// with 8 steps 16 loads per lane and strip in flight: the weights come from HBM and a wave has nothing
+// else to do meanwhile), then x, which comes from the caches, in halves of up to 4 steps.
+// k: the lane's first k of the chunk (lanes of group g take k + 16 g .. + 16 of every step).
+// w_lane, x_lane: whether this lane's row of the strip, and its token, exist: the others load nothing (one
+// condition around all loads of a kind), multiply what their registers happen to hold, and their results,
+// rows and columns of their own, are never stored.
+template <int STRIPS, int S>
+__device__ __forceinline__ void rows_chunk(const uint16_t* (&w_row)[STRIPS], const uint16_t* x_row, int k,
+                                           bool w_lane, bool x_lane, floatx4 (&acc)[STRIPS]) {
+  RowPack wa[STRIPS][S][2];
+  if (w_lane) {
+#pragma unroll
+    for (int st = 0; st < STRIPS; ++st)
+#pragma unroll
+      for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) wa[st][s][h].u = *reinterpret_cast<const uint4*>(w_row[st] + k + s * 64 + h * 8);
+  }
+  // (the compiler would rather ask for a few pieces, multiply, and ask for the next: it is told not to move
+  // anything across these lines, so that all of the chunk's weights are on their way before the first wait)
+  __builtin_amdgcn_sched_barrier(0);
+  constexpr int kHalf = S > 4 ? 4 : S;
+#pragma unroll
+  for (int first = 0; first < S; first += kHalf) {
+    RowPack xb[kHalf][2];
+    if (x_lane) {
+#pragma unroll
+      for (int s = 0; s < kHalf; ++s)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          if (first + s < S) xb[s][h].u = *reinterpret_cast<const uint4*>(x_row + k + (first + s) * 64 + h * 8);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int st = 0; st < STRIPS; ++st)
+#pragma unroll
+      for (int s = 0; s < kHalf; ++s)
+        if (first + s < S) {
+          acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[st][first + s][0].v, xb[s][0].v, acc[st], 0, 0, 0);
+          acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[st][first + s][1].v, xb[s][1].v, acc[st], 0, 0, 0);
+        }
+  }
+}
+
+// The last step of a K that is no multiple of 64 (K is one of 8): a lane whose k lies beyond K reads the
+// row's last 8 values instead and gets zeros for x.
+template <int STRIPS>
+__device__ __forceinline__ void rows_last_step(const uint16_t* (&w_row)[STRIPS], const uint16_t* x_row, int k, int k_end,
+                                               floatx4 (&acc)[STRIPS]) {
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int kk = k + h * 8, from = min(kk, k_end - 8);
+    RowPack xb;
+    xb.u = *reinterpret_cast<const uint4*>(x_row + from);
+    if (kk >= k_end) xb.u = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int st = 0; st < STRIPS; ++st) {
+      RowPack wa;
+      wa.u = *reinterpret_cast<const uint4*>(w_row[st] + from);
+      acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa.v, xb.v, acc[st], 0, 0, 0);
+    }
+  }
+}
+
 // WAVES: 2, 4, 8 or 16 waves share K (more waves for a long K or few strips, fewer when the strips
 // alone fill the chip: every wave costs a dispatch).  STRIPS: MFMA strips of 16 rows of W a
 // workgroup (2 when W has rows in plenty: each wave's part of x then serves twice the weights).
@@ -80,20 +145,19 @@ __global__ void __launch_bounds__(WAVES * 64)
 gemm_rows_kernel(const RowsArgs a) {
   __shared__ float partial[STRIPS][WAVES][64][4];   // each wave's 16 x 16 sums per strip
   __shared__ float scale_part[WAVES * 4][16];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // (the same for the wave's lanes: what depends on it alone is scalar)
   const int col = lane & 15, grp = lane >> 4;
   const int block_row = blockIdx.x * a.rows_per_block;
   const int strip_rows = STRIPS == 1 ? a.rows_per_block : 16;                 // with 8 rows a block, half the strip is idle
   const int k_begin = wave * a.k_per_wave, k_end = min(a.K, k_begin + a.k_per_wave);
-  bool row_live[STRIPS];
+  // (a row beyond the matrix, in its last strip, becomes the last row: read again, never stored)
   const uint16_t* w_row[STRIPS];
 #pragma unroll
-  for (int st = 0; st < STRIPS; ++st) {
-    row_live[st] = col < strip_rows && block_row + st * 16 + col < a.N;
+  for (int st = 0; st < STRIPS; ++st)
     w_row[st] = a.w + static_cast<size_t>(min(block_row + st * 16 + col, a.N - 1)) * a.K;
-  }
   const uint16_t* x_row = a.x + static_cast<size_t>(min(col, a.M - 1)) * a.K;
-  const bool token_live = col < a.M;
+  const bool w_lane = col < strip_rows, x_lane = col < a.M;
 
   // the norm's partial sums of squares are asked for before the weights, and added up after the
   // products: their way from the L2 is hidden behind the weights' way from memory
@@ -141,40 +205,25 @@ gemm_rows_kernel(const RowsArgs a) {
   floatx4 acc[STRIPS];
 #pragma unroll
   for (int st = 0; st < STRIPS; ++st) acc[st] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // No load stands under a lane's condition (such a load costs a dozen instructions around it, and a wave
+  // issues 24 in a row here): the wave's part of K is taken in chunks of up to 8 whole steps of 64, each
+  // chunk straight-line code for its number of steps, which is the same for all lanes; a K that is no
+  // multiple of 64 ends in a step of its own.
   for (int k0 = k_begin; k0 < k_end; k0 += 512) {
-    // 512 k of W at once (16 loads of 16 bytes per lane and strip in flight: the weights come from
-    // HBM and a wave has nothing else to do meanwhile); x, which comes from the caches, in two halves
-    RowPack wa[STRIPS][8][2];
-#pragma unroll
-    for (int st = 0; st < STRIPS; ++st)
-#pragma unroll
-      for (int s = 0; s < 8; ++s) {
-        const int k = k0 + s * 64 + grp * 16;
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-          wa[st][s][h].u = row_live[st] && k + h * 8 < k_end ? *reinterpret_cast<const uint4*>(w_row[st] + k + h * 8)
-                                                             : make_uint4(0, 0, 0, 0);
-      }
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      if (k0 + half * 256 >= k_end) break;
-      RowPack xb[4][2];
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int k = k0 + (half * 4 + s) * 64 + grp * 16;
-#pragma unroll
-        for (int h = 0; h < 2; ++h)
-          xb[s][h].u = k + h * 8 < k_end && token_live ? *reinterpret_cast<const uint4*>(x_row + k + h * 8)
-                                                       : make_uint4(0, 0, 0, 0);
-      }
-#pragma unroll
-      for (int st = 0; st < STRIPS; ++st)
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[st][half * 4 + s][0].v, xb[s][0].v, acc[st], 0, 0, 0);
-          acc[st] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[st][half * 4 + s][1].v, xb[s][1].v, acc[st], 0, 0, 0);
-        }
+    const int steps = min(8, (k_end - k0) >> 6);
+    const int k = k0 + grp * 16;
+    switch (steps) {
+      case 8: rows_chunk<STRIPS, 8>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 7: rows_chunk<STRIPS, 7>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 6: rows_chunk<STRIPS, 6>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 5: rows_chunk<STRIPS, 5>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 4: rows_chunk<STRIPS, 4>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 3: rows_chunk<STRIPS, 3>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 2: rows_chunk<STRIPS, 2>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      case 1: rows_chunk<STRIPS, 1>(w_row, x_row, k, w_lane, x_lane, acc); break;
+      default: break;
     }
+    if (steps < 8 && k0 + steps * 64 < k_end) rows_last_step<STRIPS>(w_row, x_row, k + steps * 64, k_end, acc);
   }
   // acc[st][j] = sum over this wave's k of W[block_row + st*16 + grp*4 + j][k] * x[col][k]
 #pragma unroll
