@@ -140,8 +140,11 @@ __device__ __forceinline__ void rows_last_step(const uint16_t* (&w_row)[STRIPS],
 // WAVES: 2, 4, 8 or 16 waves share K (more waves for a long K or few strips, fewer when the strips
 // alone fill the chip: every wave costs a dispatch).  STRIPS: MFMA strips of 16 rows of W a
 // workgroup (2 when W has rows in plenty: each wave's part of x then serves twice the weights).
+// With one strip a workgroup the kernel is held to the registers of 4 waves a SIMD (128): a few more, and a
+// compute unit holds 3 workgroups of 4 waves where it held 4, which the products with many strips pay for
+// (Llama-3-8B's gate/up at batch 1: 57 us against 54).
 template <int EPILOGUE, int WAVES, int STRIPS>
-__global__ void __launch_bounds__(WAVES * 64)
+__global__ void __launch_bounds__(WAVES * 64, STRIPS == 1 ? 4 : 2)
 gemm_rows_kernel(const RowsArgs a) {
   __shared__ float partial[STRIPS][WAVES][64][4];   // each wave's 16 x 16 sums per strip
   __shared__ float scale_part[WAVES * 4][16];
