@@ -47,17 +47,21 @@ class SafetensorsFile:
     def __init__(self, path: str):
         self.path = path
         try:
-            self._handle = open(path, "rb")
+            handle = open(path, "rb")
         except OSError as error:
             raise EngineError(ErrorCode.IO, f"unable to open weights: {path} ({error.strerror})") from None
-        size = os.fstat(self._handle.fileno()).st_size
+        with handle:                       # (the mapping made at the end keeps the file open by itself)
+            self._read(handle, path)
+
+    def _read(self, handle, path: str) -> None:
+        size = os.fstat(handle.fileno()).st_size
         if size < 8:
             raise _bad(f"{path}: shorter than a safetensors header")
-        (header_length,) = struct.unpack("<Q", self._handle.read(8))
+        (header_length,) = struct.unpack("<Q", handle.read(8))
         if header_length > _MAX_HEADER or 8 + header_length > size:
             raise _bad(f"{path}: header length {header_length} does not fit the file")
         try:
-            header = json.loads(self._handle.read(header_length).decode("utf-8"),
+            header = json.loads(handle.read(header_length).decode("utf-8"),
                                 object_pairs_hook=self._no_duplicates)
         except (ValueError, UnicodeDecodeError) as error:
             raise _bad(f"{path}: header is not valid JSON ({error})") from None
@@ -98,7 +102,7 @@ class SafetensorsFile:
             cursor = end
         if payload_begin + cursor != size and spans:
             raise _bad(f"{path}: {size - payload_begin - cursor} bytes after the last tensor")
-        self._map = mmap.mmap(self._handle.fileno(), 0, access=mmap.ACCESS_READ) if size > 0 else None
+        self._map = mmap.mmap(handle.fileno(), 0, access=mmap.ACCESS_READ) if size > 0 else None
 
     @staticmethod
     def _no_duplicates(pairs):
