@@ -3,6 +3,7 @@
 truncated file), on safetensors files instead of its own format."""
 import json
 import os
+import pathlib
 import struct
 
 import pytest
@@ -51,7 +52,7 @@ def test_random_model_loads_and_is_seeded(tmp_path):
     assert set(a) == {spec.name for spec in specs}
     assert all(torch.equal(a[name], b[name]) for name in a)
     assert not torch.equal(a["lm_head.weight"], c["lm_head.weight"])
-    assert json.load(open(os.path.join(one, "config.json")))["hidden_size"] == 32
+    assert json.loads(pathlib.Path(one, "config.json").read_text())["hidden_size"] == 32
     # a tensor's values depend on (seed, name) only, not on which other tensors are drawn
     alone = random_tensors([s for s in specs if s.name == "model.norm.weight"], seed=3)
     assert torch.equal(alone["model.norm.weight"], a["model.norm.weight"])
@@ -136,17 +137,17 @@ def test_broken_files(tmp_path):
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.IO
     path = str(tmp_path / "model.safetensors")
     write_safetensors(path, {"w": torch.randn(4, 4)})
-    raw = open(path, "rb").read()
-    open(path, "wb").write(raw[:-5])                                   # truncated (tests/unit_tests.cpp:166-170)
+    raw = pathlib.Path(path).read_bytes()
+    pathlib.Path(path).write_bytes(raw[:-5])                                   # truncated (tests/unit_tests.cpp:166-170)
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
-    open(path, "wb").write(raw + b"\0\0\0\0")                          # trailing bytes
+    pathlib.Path(path).write_bytes(raw + b"\0\0\0\0")                          # trailing bytes
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
-    open(path, "wb").write(raw[:4])
+    pathlib.Path(path).write_bytes(raw[:4])
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
 
     def with_header(header, payload=b"\0" * 64):
         text = json.dumps(header).encode()
-        open(path, "wb").write(struct.pack("<Q", len(text)) + text + payload)
+        pathlib.Path(path).write_bytes(struct.pack("<Q", len(text)) + text + payload)
     with_header({"w": {"dtype": "F32", "shape": [4, 4], "data_offsets": [0, 60]}})          # bytes do not fit the shape
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_SHAPE
     with_header({"w": {"dtype": "F8_E4M3", "shape": [64], "data_offsets": [0, 64]}})
@@ -154,9 +155,9 @@ def test_broken_files(tmp_path):
     with_header({"w": {"dtype": "F32", "shape": [8], "data_offsets": [0, 32]}, "v": {"dtype": "F32", "shape": [8], "data_offsets": [16, 48]}})
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT     # overlap
     text = b'{"w": {"dtype": "F32", "shape": [8], "data_offsets": [0, 32]}, "w": {"dtype": "F32", "shape": [8], "data_offsets": [32, 64]}}'
-    open(path, "wb").write(struct.pack("<Q", len(text)) + text + b"\0" * 64)
+    pathlib.Path(path).write_bytes(struct.pack("<Q", len(text)) + text + b"\0" * 64)
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT     # duplicate name
-    open(path, "wb").write(struct.pack("<Q", 1 << 40) + b"{}")
+    pathlib.Path(path).write_bytes(struct.pack("<Q", 1 << 40) + b"{}")
     assert code_of(lambda: WeightStore(str(tmp_path))).code == ErrorCode.INVALID_FORMAT
 
 
