@@ -957,7 +957,7 @@ def test_two_replays_cut_differently_agree_through_the_comparison_program(setups
     # 12 pages of 16: "a" and "b" take 5 + 3, then "a" and "c" 5 + 6, three of them the pages "b" gave back
     run = run_trace(setup, dtype, tmp_path / "cut", cut, 192, ["--check-finite"])
     assert run.returncode == 0, run.stderr
-    index = [json.loads(line) for line in open(tmp_path / "cut" / "index.jsonl")]
+    index = [json.loads(line) for line in (tmp_path / "cut" / "index.jsonl").read_text().splitlines()]
     assert len(index) == sum(len(tokens) for tokens in streams.values())
     assert {(row["id"], row["position"]) for row in index} == {(name, place) for name, tokens in streams.items() for place in range(len(tokens))}
     gate = ["--atol", "1e-5", "--rtol", "1e-5"] if dtype == "float32" else ["--atol", "0.15", "--rtol", "0.03"]
