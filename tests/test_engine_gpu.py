@@ -831,6 +831,40 @@ def test_long_prompts_take_the_walk_through_lds(tmp_path):
     engine.finish("check")
 
 
+def test_twenty_thousand_positions_cut_two_ways_and_in_both_precisions(tmp_path):
+    """A sequence of 20000 positions (1250 pages behind one block table; the plain implementation's
+    20000 x 20000 scores are out of reach, what the kernels find among so many keys is
+    tests/test_kernels_gpu.py's): the prompt in portions of 4096 and of 1000, then eight tokens one by one
+    from recordings made for 32768 positions; the logits of the last positions must not depend on the cut,
+    and bfloat16 must agree with the 32-bit path, which the plain implementation holds at shorter lengths."""
+    from tlie_amd import Engine
+    raw = dict(CONFIGS["A"], max_position_embeddings=32768, num_hidden_layers=1)
+    length, tail = 20000, 8
+    tokens = random_tokens(12, length, raw["vocab_size"])
+    places = list(range(length - tail - 4, length))
+    rows = {}
+    for dtype in DTYPES:
+        folder = make_model(tmp_path / dtype, raw, seed=41, dtype_name="bfloat16")      # (the same stored values for both)
+        engine = Engine(folder, dtype=dtype, max_tokens=2 * length + 64, page_size=16, max_requests=2)
+        replay = Replayer(engine)
+        for name, portion in (("wide", 4096), ("narrow", 1000)):
+            cursor = 0
+            while cursor < length - tail:
+                size = min(portion, length - tail - cursor)
+                wanted = [place - cursor for place in places if cursor <= place < cursor + size]
+                replay.step([(name, tokens[cursor:cursor + size], wanted)])
+                cursor += size
+            for position in range(length - tail, length):
+                replay.step([(name, [tokens[position]], [0])])
+            assert len(engine.cache.page_list(name, 0)) == length // 16
+        assert any(key[1] == 32768 for key in engine.runner._graphs), sorted(engine.runner._graphs)
+        engine.finish("wide")
+        engine.finish("narrow")
+        rows[dtype] = replay.logits_of("wide", places)
+        assert_close(replay.logits_of("narrow", places), rows[dtype], CUT_TOLERANCE[dtype], f"{dtype}: portions of 1000 against portions of 4096")
+    assert_close(rows["bfloat16"], rows["float32"].double(), TOLERANCE["bfloat16"], "bfloat16 against the 32-bit path")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_decoding_across_the_lengths_that_recordings_are_made_for(tmp_path, dtype):
     """A recording of decode steps is made for sequences up to a power of two of positions (its

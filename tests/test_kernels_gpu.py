@@ -669,6 +669,30 @@ def test_attention_mfma_over_thousands_of_keys():
             assert rel_err(got, want) < TOL["bfloat16"], f"needle {needle}: {col_tiles} groups, {waves} waves, shared {shared}, {nsplit} parts"
 
 
+def test_attention_mfma_finds_one_key_among_tens_of_thousands():
+    """33000 positions in pages of 16 (a block table of 2063 entries, 17 times the 128 that a wave keeps
+    at hand): the last token alone, as a decode step with the keys in one part and in sixteen, and the last
+    40 tokens as a portion that walks all keys through LDS; a key that stands out at the sequence's
+    start, at places where parts and table windows meet, and at its end decides the result."""
+    tokens, nq, nkv, d, page = 33000, 4, 2, 64, 16
+    torch.manual_seed(9)
+    base_k, v = torch.randn(tokens, nkv, d) * 0.1, torch.randn(tokens, nkv, d)
+    q = torch.randn(tokens, nq, d) * 0.1
+    direction = torch.zeros(d)
+    direction[7] = 1.0
+    q[tokens - 40:] += 14.0 * direction
+    for needle in (0, 2047, 2048, 2063, 16383, 16384, 20625, 32767, 32959):
+        k = base_k.clone()
+        k[needle] += 14.0 * direction
+        wanted_rows = v[needle].bfloat16().float().repeat_interleave(nq // nkv, dim=0)
+        for nsplit in (1, 16):
+            got = run_attention_mfma(q, k, v, page, None, nsplit, token_list=[tokens - 1], shuffle_seed=needle)[0].float().cpu()
+            assert (got - wanted_rows).abs().max().item() < 0.05, f"decode, needle at {needle}, {nsplit} parts: missed"
+        got = run_attention_mfma(q, k, v, page, None, 1, token_list=list(range(tokens - 40, tokens)), shuffle_seed=needle,
+                                 col_tiles=2, waves=4, shared=True).float().cpu()
+        assert (got - wanted_rows).abs().max().item() < 0.05, f"portion, needle at {needle}: missed"
+
+
 def test_attention_mfma_mixed_step():
     """Three sequences in one step: a portion of a prompt, one decoded token, a whole short prompt;
     each must equal what it gives alone."""
