@@ -9,9 +9,9 @@ import sys
 import pytest
 import torch
 
-from gpu_helpers import (CONFIGS, CUT_TOLERANCE, DTYPES, TOLERANCE, Replayer, assert_close, first_bad_row, load_plain,
+from gpu_helpers import (CONFIGS, CUT_TOLERANCE, DTYPES, TOLERANCE, Replayer, _row_errors, assert_close, first_bad_row, load_plain,
                          make_model, random_tokens)
-from plain_llama import plain_forward, plain_generate_greedy
+from plain_llama import plain_forward, plain_generate_greedy, stored_as
 from tlie_amd import ops
 
 pytestmark = pytest.mark.gpu
@@ -122,6 +122,17 @@ def test_named_intermediate_tensors_on_the_route_of_few_rows(setups, name):
     tokens = request_tokens(name, 4, 45)
     plain = {}
     plain_forward(setup["raw"], setup["weights"], tokens, trace=plain)
+    # What a tensor in the middle of the model may differ by: the tolerance of the logits, or, where 16-bit
+    # storage alone costs more than that, a quarter more than it costs: the plain implementation once more
+    # with every stored activation rounded to bfloat16 and all sums still float64 is the yardstick (what the
+    # last layer's feed-forward adds is a small difference of large numbers: 1.7e-2 of its rows' scale on
+    # configuration B, where the logits' 1.5e-2 had been passed by luck).
+    rounded = {}
+    plain_forward(setup["raw"], setup["weights"], tokens, trace=rounded, stored=stored_as(torch.bfloat16))
+
+    def allowed(key):
+        errors, scales = _row_errors(rounded[key][29:], plain[key][29:])
+        return max(TOLERANCE["bfloat16"], 1.25 * float((errors / scales).max()))
     layers = CONFIGS[name]["num_hidden_layers"]
     from tlie_amd import StepEntry
     engine.admit("t")
@@ -144,7 +155,7 @@ def test_named_intermediate_tensors_on_the_route_of_few_rows(setups, name):
     for trace in full:
         assert sorted(trace) == sorted(plain)
     for key in plain:
-        assert_close(torch.cat([trace[key] for trace in full]).cpu(), plain[key][29:], TOLERANCE["bfloat16"], "every name: " + key)
+        assert_close(torch.cat([trace[key] for trace in full]).cpu(), plain[key][29:], allowed(key), "every name: " + key)
     assert_close(torch.cat([trace["logits"] for trace in full]).cpu(), torch.cat([trace["logits"] for trace in traces]).cpu().double(),
                  CUT_TOLERANCE["bfloat16"], "the two routes' logits")
     names = ["embedding"] + [f"layer{layer}.{part}" for layer in range(layers) for part in ("attention_output", "mlp_output", "output")] \
@@ -154,7 +165,7 @@ def test_named_intermediate_tensors_on_the_route_of_few_rows(setups, name):
     for key in names:
         got = torch.cat([trace[key] for trace in traces]).cpu()
         assert got.dtype == torch.float32 and got.shape == plain[key][29:].shape, key
-        assert_close(got, plain[key][29:], TOLERANCE["bfloat16"], key)
+        assert_close(got, plain[key][29:], allowed(key), key)
     # the same steps without a trace (replayed from recordings): the same logits up to the cut's tolerance
     engine.admit("u")
     engine.step([StepEntry("u", tokens[:29], [])])
