@@ -675,7 +675,8 @@ def test_seeded_sampling_is_the_same_under_every_cut_and_under_preemption(setups
     # 8 pages of 16 positions: the three requests need 2 + 4 + 6 at their ends, so they cannot all stay
     tight = Engine(setup["folder"], dtype=dtype, max_tokens=128, page_size=16, max_requests=4)
     assert tight.cache.num_pages == 8
-    scheduler = Scheduler(tight.cache, max_tokens_per_step=24, max_seqs_per_step=4, chunk_size=16,
+    # (admitted as soon as a first portion fits, so that all three are in at once and the last must give way)
+    scheduler = Scheduler(tight.cache, max_tokens_per_step=24, max_seqs_per_step=4, chunk_size=16, admit_partial=True,
                           max_positions=tight.spec.max_positions, eos_token_id=tight.spec.eos_token_id)
     requests = [Request(id=("tight", i), prompt=list(prompt),
                         params=SamplingParams(max_tokens=new_tokens, temperature=temperature, top_p=top_p, seed=seed + i))
@@ -1042,10 +1043,11 @@ def test_several_prompts_from_the_command_line_batched_in_portions_with_preempti
     listed = tmp_path / "prompts.txt"
     listed.write_text("ids:" + " ".join(str(token) for token in prompts[2]) + "\n")
     # the prompts take 2 pages of 16 each; with 28 more positions each grows into a third (and a fourth):
-    # 7 pages hold the three prompts, and not what they grow to
+    # 7 pages hold the three prompts, and not what they grow to (all three are admitted at once:
+    # --admit-partial; by default the third would wait until the pool has room for all of it)
     run = subprocess.run(cli + ["generate", setup["folder"], text, "28", "--dtype", "float32", "--prompts-file", str(listed),
                                 "--page-size", "16", "--max-cache-tokens", "112", "--chunk-size", "16", "--max-tokens-per-step", "24",
-                                "--max-requests", "3"], capture_output=True, text=True, timeout=300)
+                                "--max-requests", "3", "--admit-partial"], capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr
     result = json.loads(run.stdout)
     assert [row["generated_tokens"] for row in result["requests"]] == want

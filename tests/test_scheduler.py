@@ -143,8 +143,9 @@ def test_requests_that_can_never_fit_are_refused():
 
 def test_pages_run_out_while_decoding_the_last_admitted_is_preempted():
     # 6 pages of 4: two requests of 9-token prompts take 3 pages each (positions 0..11); when they
-    # grow past 12 positions each needs a fourth page and none is free.
-    cache, scheduler = make(num_pages=6, page_size=4)
+    # grow past 12 positions each needs a fourth page and none is free.  (Admitted as soon as a first
+    # portion fits: by default the second would wait for the first to finish, see below.)
+    cache, scheduler = make(num_pages=6, page_size=4, admit_partial=True)
     a = Request("a", list(range(1, 10)), SamplingParams(max_tokens=8))
     b = Request("b", list(range(21, 30)), SamplingParams(max_tokens=8))
     scheduler.add(a)
@@ -167,7 +168,7 @@ def test_a_preempted_request_returns_its_tokens_to_the_steps_budget():
     step's rotation: when the second one finds no page and preempts it, the token it had in the plan is
     free again, so the step still takes the other two (the budget is not charged for a request that
     left the plan)."""
-    cache, scheduler = make(num_pages=6, page_size=4, max_tokens_per_step=3)
+    cache, scheduler = make(num_pages=6, page_size=4, max_tokens_per_step=3, admit_partial=True)
     requests = [Request(name, list(range(base, base + 7)), SamplingParams(max_tokens=8))
                 for name, base in (("a", 1), ("b", 11), ("c", 21))]
     for request in requests:
@@ -199,7 +200,7 @@ def test_budget_after_preemption_is_what_the_plan_holds():
 def test_prompts_that_block_each_other_are_untangled():
     # two prompts of 28 tokens (7 pages each) in a pool of 10: cut into portions of 8 they take
     # pages turn by turn until neither can go on; the later one is preempted, the earlier finishes.
-    cache, scheduler = make(num_pages=10, page_size=4, max_tokens_per_step=16, chunk_size=8)
+    cache, scheduler = make(num_pages=10, page_size=4, max_tokens_per_step=16, chunk_size=8, admit_partial=True)
     a = Request("a", list(range(1, 29)), SamplingParams(max_tokens=2))
     b = Request("b", list(range(31, 59)), SamplingParams(max_tokens=2))
     scheduler.add(a)
@@ -207,6 +208,58 @@ def test_prompts_that_block_each_other_are_untangled():
     drive(cache, scheduler)
     assert a.generated == expected_output(a.prompt, 2) and b.generated == expected_output(b.prompt, 2)
     assert b.preemptions >= 1 and a.preemptions == 0
+
+
+def test_a_waiting_request_is_admitted_when_all_it_brings_fits():
+    # the same two prompts of 7 pages each in a pool of 10: by default the second is not admitted for a
+    # first portion that would then fight the first for pages; it waits until the first has finished
+    cache, scheduler = make(num_pages=10, page_size=4, max_tokens_per_step=16, chunk_size=8)
+    a = Request("a", list(range(1, 29)), SamplingParams(max_tokens=2))
+    b = Request("b", list(range(31, 59)), SamplingParams(max_tokens=2))
+    scheduler.add(a)
+    scheduler.add(b)
+    log = []
+    drive(cache, scheduler, log)
+    assert a.generated == expected_output(a.prompt, 2) and b.generated == expected_output(b.prompt, 2)
+    assert scheduler.stats["preemptions"] == 0
+    last_of_a = max(index for index, step in enumerate(log) if any(rid == "a" for rid, _, _, _ in step))
+    first_of_b = min(index for index, step in enumerate(log) if any(rid == "b" for rid, _, _, _ in step))
+    assert first_of_b > last_of_a
+    # with room for both (7 + 7 pages, a page of growth each and one to spare) they run side by side
+    cache, scheduler = make(num_pages=17, page_size=4, max_tokens_per_step=16, chunk_size=8)
+    a = Request("a", list(range(1, 29)), SamplingParams(max_tokens=2))
+    b = Request("b", list(range(31, 59)), SamplingParams(max_tokens=2))
+    scheduler.add(a)
+    scheduler.add(b)
+    log = []
+    drive(cache, scheduler, log)
+    assert any({rid for rid, _, _, _ in step} == {"a", "b"} for step in log) and scheduler.stats["preemptions"] == 0
+    # a request alone is admitted whatever it needs (`add` has refused what the pool could never hold)
+    cache, scheduler = make(num_pages=8, page_size=4)
+    alone = Request("x", list(range(1, 29)), SamplingParams(max_tokens=4))
+    scheduler.add(alone)
+    drive(cache, scheduler)
+    assert alone.generated == expected_output(alone.prompt, 4)
+
+
+def test_requests_that_outnumber_the_pool_many_times():
+    """Twenty requests of 21 to 40 prompt tokens and 12 outputs on a pool of 30 pages of 4 (three of
+    them at a time): the outputs are those of undisturbed runs under either way of admitting; admitted
+    whole, requests are preempted only when those that run outgrow the page of growth kept for each, a
+    fraction of what admitting first portions costs."""
+    counts = {}
+    for partial in (False, True):
+        cache, scheduler = make(num_pages=30, page_size=4, max_requests=8, max_tokens_per_step=32, admit_partial=partial)
+        requests = [Request(f"r{i}", [(7 * i + j) % 50 + 1 for j in range(21 + i)], SamplingParams(max_tokens=12)) for i in range(20)]
+        for request in requests:
+            scheduler.add(request)
+        drive(cache, scheduler, max_steps=5000)
+        for request in requests:
+            assert request.generated == expected_output(request.prompt, 12)
+        assert cache.free_pages() == [30] and cache.free_slots == 8
+        counts[partial] = (scheduler.stats["preemptions"], scheduler.stats["prefill_tokens"])
+    assert counts[True][0] >= 10 and counts[False][0] * 3 <= counts[True][0], counts
+    assert counts[False][1] < counts[True][1]              # and fewer prompt tokens run twice
 
 
 def test_more_decoders_than_the_budget_rotate():

@@ -20,7 +20,8 @@ Options (after the positionals): --dtype bfloat16|float32, --temperature T, --to
 scheduler: --max-cache-tokens N (positions the page pool holds), --page-size P, --max-requests R
 (request slots), --max-tokens-per-step T (a step's token budget), --chunk-size C (the most tokens of
 one prompt in a step), --prompt-tokens-beside-decodes N (the most prompt tokens in a step that also
-decodes); `batch`: --batch N (default 4), --min-ratio X (fail below this speed-up).
+decodes), --admit-partial (a waiting request is admitted as soon as a first portion of it fits the pool,
+not only when all of it does); `batch`: --batch N (default 4), --min-ratio X (fail below this speed-up).
 """
 from __future__ import annotations
 
@@ -38,7 +39,7 @@ USAGE = ("usage: tinyllama_amd generate MODEL_DIR PROMPT MAX_TOKENS [GOLDEN_JSON
          "       tinyllama_amd random MODEL_DIR CONFIG_JSON SEED\n"
          "options: [--dtype bfloat16|float32] [--temperature T] [--top-p P] [--seed S] [--expect-sha256 HEX]\n"
          "         [--max-cache-tokens N] [--page-size P] [--max-requests R] [--max-tokens-per-step T] [--chunk-size C]\n"
-         "         [--prompt-tokens-beside-decodes N] [--prompts-file FILE] [--batch N] [--min-ratio X]\n")
+         "         [--prompt-tokens-beside-decodes N] [--admit-partial] [--prompts-file FILE] [--batch N] [--min-ratio X]\n")
 
 
 def parse_integer(text: str, name: str, minimum: int) -> int:
@@ -116,7 +117,8 @@ def command_generate(args) -> int:
     outputs = engine.generate(prompts, max_tokens=max_tokens, temperature=args.temperature, top_p=args.top_p,
                               seed=args.seed, timings=timings, stats=stats,
                               max_tokens_per_step=args.max_tokens_per_step or 2048, chunk_size=args.chunk_size or None,
-                              prompt_tokens_beside_decodes=args.prompt_tokens_beside_decodes or None)
+                              prompt_tokens_beside_decodes=args.prompt_tokens_beside_decodes or None,
+                              admit_partial=args.admit_partial)
     generated = outputs[0]
     elapsed = (time.perf_counter() - started) * 1e3
     if len(args.rest) > 1:
@@ -323,6 +325,7 @@ def main(argv=None) -> int:
     parser.add_argument("--max-tokens-per-step", type=int, default=0)
     parser.add_argument("--chunk-size", type=int, default=0)
     parser.add_argument("--prompt-tokens-beside-decodes", type=int, default=0)
+    parser.add_argument("--admit-partial", action="store_true")
     parser.add_argument("--prompts-file", default=None)
     parser.add_argument("--batch", type=int, default=4)
     parser.add_argument("--min-ratio", type=float, default=0.0)

@@ -128,7 +128,7 @@ class Engine:
                  top_p: float = 1.0, seed: int = 0, stop_on_eos: bool = False, max_tokens_per_step: int = 2048,
                  max_seqs_per_step: int | None = None, chunk_size: int | None = None,
                  timings: dict | None = None, stats: dict | None = None,
-                 prompt_tokens_beside_decodes: int | None = None) -> list[list[int]]:
+                 prompt_tokens_beside_decodes: int | None = None, admit_partial: bool = False) -> list[list[int]]:
         """Token ids in, generated token ids out, one list per prompt.  Request i samples with
         seed + i.  All prompts run together under the scheduler (continuous batching, prompts cut
         into portions under the token budget).  `timings`: a dict that receives the sums of the
@@ -136,11 +136,11 @@ class Engine:
         only decode (the keys of the reference's `generate`, app/cuda_reference.cu:216-224).
         `stats`: a dict that receives what the scheduler counted (steps, prompt and decoded tokens,
         preemptions) and how many matrix products of this process fell from the vendor's library to the
-        plain kernel (`library_fallbacks`).  prompt_tokens_beside_decodes: see `Scheduler`."""
+        plain kernel (`library_fallbacks`).  prompt_tokens_beside_decodes, admit_partial: see `Scheduler`."""
         scheduler = Scheduler(self.cache, max_tokens_per_step=max_tokens_per_step,
                               max_seqs_per_step=max_seqs_per_step or self.cache.max_requests, chunk_size=chunk_size,
                               max_positions=self.spec.max_positions, eos_token_id=self.spec.eos_token_id,
-                              prompt_tokens_beside_decodes=prompt_tokens_beside_decodes)
+                              prompt_tokens_beside_decodes=prompt_tokens_beside_decodes, admit_partial=admit_partial)
         requests = []
         for index, prompt in enumerate(prompts):
             params = SamplingParams(max_tokens=max_tokens, temperature=temperature, top_p=top_p, seed=seed + index,
